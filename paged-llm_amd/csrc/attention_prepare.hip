@@ -4,7 +4,7 @@
 //   attn_prepare      per token and head, from the float sums of the q/k/v product: + bias, a short causal convolution
 //                     over time on every channel (inputs of earlier steps from the request's state slot), rotary
 //                     encoding of the first rot elements of q and k heads (pairs (i, i + rot/2) or (2i, 2i + 1)),
-//                     q and k divided by their root mean square over the head, q written as rows of padded heads,
+//                     q and k divided by their root mean square over the head (unless qk_norm is 0), q written as rows of padded heads,
 //                     k and v written into their cache pages;
 //   conv_inputs_keep  leaves the last taps - 1 projected rows of every sequence in its state slot;
 //   gate_heads        out[t, h, :dv] = o[t, h, :dv] * sigmoid(gate[t, h]) from padded heads to packed ones.
@@ -29,7 +29,7 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
     const float* __restrict__ proj, int ld, const float* __restrict__ bias, const float* __restrict__ conv_w, int taps,
     const float* __restrict__ state, size_t slot_stride, const int* __restrict__ state_slots, const int* __restrict__ seq_starts,
     const int* __restrict__ cu_seqlens, int num_seqs, const int* __restrict__ positions, const float* __restrict__ cos_table,
-    const float* __restrict__ sin_table, int rot, int interleaved, float eps, int heads, int kv_heads, int d, int dv, int D,
+    const float* __restrict__ sin_table, int rot, int interleaved, float eps, int qk_norm, int heads, int kv_heads, int d, int dv, int D,
     T* __restrict__ q_out, const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int block_size) {
   __shared__ float vals[kPrepMaxHead];
   const int lane = threadIdx.x;
@@ -100,9 +100,11 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
       }
       if (e < width) sq = fmaf(x[r], x[r], sq);
     }
-    const float inv = 1.f / sqrtf(wave_sum(sq) / (float)width + eps);
+    if (qk_norm) {
+      const float inv = 1.f / sqrtf(wave_sum(sq) / (float)width + eps);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) x[r] *= inv;
+      for (int r = 0; r < 4; ++r) x[r] *= inv;
+    }
   }
   if (kind == 0) {
     T* out = q_out + ((size_t)tok * heads + head) * D;
@@ -163,7 +165,7 @@ __global__ __launch_bounds__(256) void conv_inputs_keep_kernel(
 PLLM_API int pllm_attn_prepare(int dtype, const float* proj, int ld, const float* bias, const float* conv_w, int taps, float* state,
                                long slot_stride, const int* state_slots, const int* seq_starts, const int* cu_seqlens, int num_seqs,
                                const int* positions, const float* cos_table, const float* sin_table, int rot, int interleaved,
-                               float eps, int heads, int kv_heads, int d, int dv, int D, void* q_out, const int* slot_mapping,
+                               float eps, int qk_norm, int heads, int kv_heads, int d, int dv, int D, void* q_out, const int* slot_mapping,
                                void* k_pages, void* v_pages, int block_size, int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || dv <= 0 || d > D || dv > D || D > kPrepMaxHead || rot < 0 || rot > d || (rot & 1) || taps > kPrepMaxTaps) return -2;
@@ -173,7 +175,7 @@ PLLM_API int pllm_attn_prepare(int dtype, const float* proj, int ld, const float
   dim3 grid(num_tokens, heads + (write ? 2 * kv_heads : 0)), block(64);
 #define PLLM_PREP(T)                                                                                                              \
   hipLaunchKernelGGL(attn_prepare_kernel<T>, grid, block, 0, stream, proj, ld, bias, conv_w, taps, state, (size_t)slot_stride,   \
-                     state_slots, seq_starts, cu_seqlens, num_seqs, positions, cos_table, sin_table, rot, interleaved, eps, heads, \
+                     state_slots, seq_starts, cu_seqlens, num_seqs, positions, cos_table, sin_table, rot, interleaved, eps, qk_norm, heads, \
                      kv_heads, d, dv, D, (T*)q_out, slot_mapping, (T*)k_pages, (T*)v_pages, block_size)
   if (dtype == PLLM_F32) PLLM_PREP(float); else PLLM_PREP(bf16);
 #undef PLLM_PREP

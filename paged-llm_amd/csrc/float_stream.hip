@@ -372,3 +372,65 @@ PLLM_API int pllm_place_rows(int out_dtype, const float* x, void* out, long out_
   else hipLaunchKernelGGL(place_rows_kernel<bf16>, grid, block, 0, stream, x, (bf16*)out, out_stride, hidden);
   PLLM_RETURN_LAST_ERROR();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Dynamic tanh, a norm that computes no statistics, y = tanh(alpha x) * w + b element by element, around a float stream:
+//   branch given:  stream[r] += branch[r] in place (no row_index then);
+//   rows given:    rows[r] = T(tanh(alpha * stream[src]) * w + b), src = row_index[r] or r, with the stream as it is
+//                  after the sum.
+// One workgroup per row; four elements per thread and load where `vec` says the rows allow it (hidden a multiple of 4,
+// rows on 16-byte boundaries in float and 8-byte ones in T).
+template <typename TO>
+__global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ branch, float* stream, const int* __restrict__ row_index,
+                                                  float alpha, const float* __restrict__ w, const float* __restrict__ b,
+                                                  TO* __restrict__ rows, long rows_stride, int hidden, int vec) {
+  const int r = blockIdx.x;
+  const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
+  float* x = stream + src * hidden;
+  const float* d = branch ? branch + (size_t)r * hidden : nullptr;
+  TO* out = rows ? rows + (size_t)r * rows_stride : nullptr;
+  if (vec) {
+    for (int i = 4 * threadIdx.x; i < hidden; i += 4 * blockDim.x) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (d) {
+        const float4 e = *reinterpret_cast<const float4*>(d + i);
+        v.x += e.x; v.y += e.y; v.z += e.z; v.w += e.w;
+        *reinterpret_cast<float4*>(x + i) = v;
+      }
+      if (out) {
+        const float4 ww = *reinterpret_cast<const float4*>(w + i), bb = *reinterpret_cast<const float4*>(b + i);
+        Quad<TO> o;
+        o.v[0] = from_f32<TO>(fmaf(tanhf(alpha * v.x), ww.x, bb.x));
+        o.v[1] = from_f32<TO>(fmaf(tanhf(alpha * v.y), ww.y, bb.y));
+        o.v[2] = from_f32<TO>(fmaf(tanhf(alpha * v.z), ww.z, bb.z));
+        o.v[3] = from_f32<TO>(fmaf(tanhf(alpha * v.w), ww.w, bb.w));
+        *reinterpret_cast<Quad<TO>*>(out + i) = o;
+      }
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = x[i];
+    if (d) {
+      v += d[i];
+      x[i] = v;
+    }
+    if (out) out[i] = from_f32<TO>(fmaf(tanhf(alpha * v), w[i], b[i]));
+  }
+}
+
+PLLM_API int pllm_dyt(int out_dtype, const float* branch, float* stream, const int* row_index, float alpha, const float* w,
+                      const float* b, void* rows, long rows_stride, int num_rows, int hidden, hipStream_t stream_) {
+  if (num_rows <= 0) return 0;
+  if (branch && row_index) return -2;
+  if (rows && (!w || !b)) return -2;
+  const size_t out_bytes = out_dtype == PLLM_F32 ? 4 : 2;
+  const int vec = hidden % 4 == 0 && ((uintptr_t)stream & 15) == 0 && (!branch || ((uintptr_t)branch & 15) == 0) &&
+                  (!rows || (((uintptr_t)rows % (4 * out_bytes)) == 0 && rows_stride % 4 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)b & 15) == 0));
+  dim3 grid(num_rows), block(hidden >= 1024 ? 256 : (hidden >= 256 ? 64 * ((hidden / 4 + 63) / 64) : 64));
+  if (out_dtype == PLLM_F32)
+    hipLaunchKernelGGL(dyt_kernel<float>, grid, block, 0, stream_, branch, stream, row_index, alpha, w, b, (float*)rows, rows_stride, hidden, vec);
+  else
+    hipLaunchKernelGGL(dyt_kernel<bf16>, grid, block, 0, stream_, branch, stream, row_index, alpha, w, b, (bf16*)rows, rows_stride, hidden, vec);
+  PLLM_RETURN_LAST_ERROR();
+}

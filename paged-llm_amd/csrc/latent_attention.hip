@@ -23,20 +23,23 @@
 
 using namespace pllm;
 
-// rows [T, row_stride]: heads x [plain | rot] of the queries at column 0, then the down-projection [rank | rot] at
-// column `down_at`.  q_out [T, heads, width]: columns rank .. rank + rot of every head receive its rotated part and the
-// columns behind them zeros (columns 0 .. rank are another kernel's).
-template <typename T>
+// rows [T, row_stride] (type TI: the pages' type T, or float sums of the product that made them): heads x [plain | rot] of
+// the queries at column 0, then the down-projection [rank | rot] at column `down_at`.  q_out [T, heads, width]: columns
+// rank .. rank + rot of every head receive its rotated part and the columns behind them zeros (columns 0 .. rank are
+// another kernel's).  rot may be 0: a latent without a rotated part (the queries' columns are not read then).
+// With q_rank > 0 the rows also hold a latent of the queries at column q_at: cq_out [T, q_rank] receives its RMS norm
+// times q_norm_w (the operand of the product that expands it into the heads' queries).
+template <typename TI, typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(
-    const T* __restrict__ rows, int row_stride, int down_at, const int* __restrict__ positions, const float* __restrict__ cos_t,
+    const TI* __restrict__ rows, int row_stride, int down_at, const int* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const float* __restrict__ norm_w, float eps, const int* __restrict__ slots,
     T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out, int heads, int plain, int rot, int rank,
-    int width, int block_size, int interleaved) {
+    int width, int block_size, int interleaved, int q_at, int q_rank, const float* __restrict__ q_norm_w, T* __restrict__ cq_out) {
   __shared__ float scratch[16];
   const int tok = blockIdx.x;
-  const T* row = rows + (size_t)tok * row_stride;
+  const TI* row = rows + (size_t)tok * row_stride;
   const int half = rot / 2;
-  const size_t table = (size_t)positions[tok] * half;
+  const size_t table = half ? (size_t)positions[tok] * half : 0;
   const int slot = slots ? slots[tok] : -1;
   T* k_row = k_pages + (size_t)(slot < 0 ? 0 : slot) * width;
   T* v_col = v_pages ? v_pages + ((size_t)(slot < 0 ? 0 : slot / block_size) * width) * block_size + (slot < 0 ? 0 : slot % block_size) : nullptr;
@@ -54,10 +57,20 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
       if (v_col) v_col[(size_t)i * block_size] = c;
     }
   }
+  if (q_rank > 0) {
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
+      const float v = to_f32(row[q_at + i]);
+      sq = fmaf(v, v, sq);
+    }
+    const float inv_q = 1.f / sqrtf(block_sum(sq, scratch) / (float)q_rank + eps);
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+      cq_out[(size_t)tok * q_rank + i] = from_f32<T>(to_f32(row[q_at + i]) * inv_q * q_norm_w[i]);
+  }
   // rotated parts: pair j of the shared key part (unit == heads) and of every head's query part
   for (int idx = threadIdx.x; idx < (heads + 1) * half; idx += blockDim.x) {
     const int unit = idx / half, j = idx % half;
-    const T* part = unit == heads ? row + down_at + rank : row + (size_t)unit * (plain + rot) + plain;
+    const TI* part = unit == heads ? row + down_at + rank : row + (size_t)unit * (plain + rot) + plain;
     const int lo_at = interleaved ? 2 * j : j, hi_at = interleaved ? 2 * j + 1 : j + half;
     float lo, hi;
     rotate_pair(to_f32(part[lo_at]), to_f32(part[hi_at]), cos_t[table + j], sin_t[table + j], lo, hi);
@@ -72,21 +85,26 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     q_out[((size_t)tok * heads + idx / pad) * width + rank + rot + idx % pad] = from_f32<T>(0.f);
 }
 
-PLLM_API int pllm_latent_prepare(int dtype, const void* rows, int row_stride, int down_at, const int* positions, const float* cos_t,
-                                 const float* sin_t, const float* norm_w, float eps, const int* slots, void* k_pages,
+// rows_dtype: the type of `rows` (the pages' type `dtype`, or float).
+PLLM_API int pllm_latent_prepare(int dtype, int rows_dtype, const void* rows, int row_stride, int down_at, const int* positions,
+                                 const float* cos_t, const float* sin_t, const float* norm_w, float eps, const int* slots, void* k_pages,
                                  void* v_pages, void* q_out, int num_tokens, int heads, int plain, int rot, int rank, int width,
-                                 int block_size, int interleaved, hipStream_t stream) {
+                                 int block_size, int interleaved, int q_at, int q_rank, const float* q_norm_w, void* cq_out,
+                                 hipStream_t stream) {
   if (num_tokens <= 0) return 0;
-  if (rot <= 0 || rot % 2 || rank <= 0 || heads <= 0 || plain < 0 || width < rank + rot || block_size <= 0) return -2;
+  if (rot < 0 || rot % 2 || rank <= 0 || heads <= 0 || plain < 0 || width < rank + rot || block_size <= 0) return -2;
+  if (rot > 0 && (!cos_t || !sin_t)) return -2;
+  if (q_rank < 0 || (q_rank > 0 && (!q_norm_w || !cq_out))) return -2;
+  if (rows_dtype != dtype && rows_dtype != PLLM_F32) return -2;
   dim3 grid(num_tokens), block(256);
-  if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, block, 0, stream, (const float*)rows, row_stride, down_at, positions, cos_t,
-                       sin_t, norm_w, eps, slots, (float*)k_pages, (float*)v_pages, (float*)q_out, heads, plain, rot, rank, width,
-                       block_size, interleaved);
-  else
-    hipLaunchKernelGGL(latent_prepare_kernel<bf16>, grid, block, 0, stream, (const bf16*)rows, row_stride, down_at, positions, cos_t,
-                       sin_t, norm_w, eps, slots, (bf16*)k_pages, (bf16*)v_pages, (bf16*)q_out, heads, plain, rot, rank, width,
-                       block_size, interleaved);
+#define PLLM_LP(TI, T)                                                                                                             \
+  hipLaunchKernelGGL((latent_prepare_kernel<TI, T>), grid, block, 0, stream, (const TI*)rows, row_stride, down_at, positions, cos_t, \
+                     sin_t, norm_w, eps, slots, (T*)k_pages, (T*)v_pages, (T*)q_out, heads, plain, rot, rank, width, block_size,    \
+                     interleaved, q_at, q_rank, q_norm_w, (T*)cq_out)
+  if (dtype == PLLM_F32) PLLM_LP(float, float);
+  else if (rows_dtype == PLLM_F32) PLLM_LP(float, bf16);
+  else PLLM_LP(bf16, bf16);
+#undef PLLM_LP
   PLLM_RETURN_LAST_ERROR();
 }
 

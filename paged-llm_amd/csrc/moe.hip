@@ -25,11 +25,14 @@ constexpr int kRouteThreads = 1024, kRoutePieces = 16;   // threads of a workgro
 
 template <typename T, int TOK>
 __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ router_w,
-                                                                  const float* __restrict__ correction, int num_tokens, int width, int n,
-                                                                  int groups, int keep, int top, int segments, int* __restrict__ ids,
-                                                                  float* __restrict__ weights) {
+                                                                  const float* __restrict__ correction, int num_tokens, int width, int n_all,
+                                                                  int extra, int scoring, int groups, int keep, int top, int segments,
+                                                                  int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ extras) {
   extern __shared__ float lds[];
-  const int per_token = 2 * n + groups + segments * n;       // floats of LDS that one token has
+  // n_all rows of the router matrix: the first n = n_all - extra are the experts' (scores, the choice), the last `extra`
+  // are further outputs of the same product that go to `extras` [tokens, extra] as they are
+  const int n = n_all - extra;
+  const int per_token = 2 * n_all + groups + segments * n_all;       // floats of LDS that one token has
   const int t0 = blockIdx.x * TOK;                           // this workgroup's tokens: t0 .. t0 + TOK - 1
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row[TOK];
@@ -41,7 +44,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
   // that the experts' weights have pushed out of the caches since the last layer: what counts is how few loads wait for
   // one another; many tokens: a router element is fetched once for TOK of them).  A router output is the sum of its
   // parts in ascending order, each part summed lane by lane and then over the wavefront, whatever TOK is.
-  const int batches = (n + 7) / 8;
+  const int batches = (n_all + 7) / 8;
   const int seg = ((width + segments - 1) / segments + 63) & ~63;
   for (int piece = wave; piece < batches * segments; piece += (int)(blockDim.x >> 6)) {
     const int e0 = (piece / segments) * 8, sg = piece % segments;
@@ -52,7 +55,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 #pragma unroll
       for (int k = 0; k < TOK; ++k) acc[j][k] = 0.f;
     const float* w = router_w + (size_t)e0 * width;
-    if (TOK == 1 && e0 + 8 <= n) {
+    if (TOK == 1 && e0 + 8 <= n_all) {
       // every load of eight elements' worth asked for before the first sum: 72 loads under way, one trip to memory
       for (int i0 = from + lane; i0 < to; i0 += 8 * 64) {
         float x[8], wv[8][8];
@@ -68,7 +71,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 #pragma unroll
           for (int j = 0; j < 8; ++j) acc[j][0] = fmaf(x[u], wv[u][j], acc[j][0]);
       }
-    } else if (e0 + 8 <= n) {
+    } else if (e0 + 8 <= n_all) {
 #pragma unroll(TOK >= 8 ? 1 : 2)
       for (int i = from + lane; i < to; i += 64) {
         float x[TOK];
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
         for (int k = 0; k < TOK; ++k) x[k] = to_f32(row[k][i]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-          if (e0 + j < n) {
+          if (e0 + j < n_all) {
             const float wj = w[(size_t)j * width + i];
 #pragma unroll
             for (int k = 0; k < TOK; ++k) acc[j][k] = fmaf(x[k], wj, acc[j][k]);
@@ -100,24 +103,25 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 #pragma unroll
       for (int k = 0; k < TOK; ++k) {
         const float total = wave_sum(acc[j][k]);
-        if (lane == 0 && e0 + j < n) lds[k * per_token + 2 * n + groups + sg * n + e0 + j] = total;
+        if (lane == 0 && e0 + j < n_all) lds[k * per_token + 2 * n_all + groups + sg * n_all + e0 + j] = total;
       }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < TOK * n; i += blockDim.x) {
-    const int k = i / n, e = i - k * n;
-    const float* part = lds + k * per_token + 2 * n + groups;
+  for (int i = threadIdx.x; i < TOK * n_all; i += blockDim.x) {
+    const int k = i / n_all, e = i - k * n_all;
+    const float* part = lds + k * per_token + 2 * n_all + groups;
     float total = part[e];
-    for (int sg = 1; sg < segments; ++sg) total += part[sg * n + e];
-    lds[k * per_token + e] = total;
+    for (int sg = 1; sg < segments; ++sg) total += part[sg * n_all + e];
+    if (e < n) lds[k * per_token + e] = total;
+    else if (t0 + k < num_tokens) extras[(size_t)(t0 + k) * extra + (e - n)] = total;
   }
   __syncthreads();
   // The choice: wavefront k makes token t0 + k's (the others keep them company at the barriers).
   const int t = t0 + wave;
   const bool chooser = wave < TOK && t < num_tokens;
   float* score = lds + (wave < TOK ? wave : 0) * per_token;   // [n]  router outputs, then scores
-  float* choice = score + n;                                  // [n]  score + correction, -inf once taken or shut out
-  float* mark = score + 2 * n;                                // [groups]
+  float* choice = score + n_all;                              // [n]  score + correction, -inf once taken or shut out
+  float* mark = score + 2 * n_all;                            // [groups]
   // Lane l looks after router outputs l, l + 64, ...; a largest element is found by a maximum over the wavefront and
   // then the lowest index that holds it (ties: the lower index wins).
   auto lowest_at = [&](const float* values, int count) {
@@ -129,7 +133,14 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
       if (values[e] == best) { at = (float)e; break; }
     return (int)(-wave_max(-at));
   };
-  if (chooser) {
+  if (chooser && scoring == 1) {
+    // scores by a sigmoid of every router output on its own
+    for (int e = lane; e < n; e += 64) {
+      const float sc = 1.f / (1.f + expf(-score[e]));
+      score[e] = sc;
+      choice[e] = sc + (correction ? correction[e] : 0.f);
+    }
+  } else if (chooser) {
     float m = -INFINITY;
     for (int e = lane; e < n; e += 64) m = fmaxf(m, score[e]);
     m = wave_max(m);
@@ -179,22 +190,26 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
   }
 }
 
+// n_all = n + extra rows of the router matrix; scoring 0: softmax over the n router outputs, 1: a sigmoid of each.
 PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* router_w, const float* correction, int num_tokens, int width,
-                            int n, int groups, int keep, int top, int* ids, float* weights, hipStream_t stream) {
+                            int n_all, int extra, int scoring, int groups, int keep, int top, int* ids, float* weights, float* extras,
+                            hipStream_t stream) {
   if (num_tokens <= 0) return 0;
+  const int n = n_all - extra;
+  if (extra < 0 || (extra > 0 && !extras) || scoring < 0 || scoring > 1) return -2;
   if (n <= 0 || groups <= 0 || n % groups || keep <= 0 || keep > groups || top <= 0 || top > (n / groups) * keep) return -2;
   // as many parts of the row as make 16 pieces (1, 2, 4, 8 or 16 parts), none shorter than 64 elements: by the router's
   // shape alone, so that a token's scores do not depend on the step it is in
   int segments = 1;
-  while (segments < kRoutePieces && ((n + 7) / 8) * segments < kRoutePieces && width / (2 * segments) >= 64) segments *= 2;
-  const size_t lds_one = (size_t)(2 * n + groups + segments * n) * sizeof(float);
+  while (segments < kRoutePieces && ((n_all + 7) / 8) * segments < kRoutePieces && width / (2 * segments) >= 64) segments *= 2;
+  const size_t lds_one = (size_t)(2 * n_all + groups + segments * n_all) * sizeof(float);
   // tokens to a workgroup (one wavefront each for the choice): 8 in steps of 512 tokens and more, 4 from 128 on, else one
   // token to sixteen wavefronts
   const int tok = (num_tokens >= 512 && 8 * lds_one <= 48 * 1024) ? 8 : (num_tokens >= 128 && 4 * lds_one <= 48 * 1024) ? 4 : 1;
   const size_t lds = lds_one * tok;
 #define PLLM_ROUTE(T, TOK, THREADS)                                                                                              \
   hipLaunchKernelGGL((moe_route_kernel<T, TOK>), dim3((num_tokens + TOK - 1) / TOK), dim3(THREADS), lds, stream, (const T*)h, ld, \
-                     router_w, correction, num_tokens, width, n, groups, keep, top, segments, ids, weights)
+                     router_w, correction, num_tokens, width, n_all, extra, scoring, groups, keep, top, segments, ids, weights, extras)
   if (dtype == PLLM_F32) { if (tok == 8) PLLM_ROUTE(float, 8, 512); else if (tok == 4) PLLM_ROUTE(float, 4, 256); else PLLM_ROUTE(float, 1, kRouteThreads); }
   else { if (tok == 8) PLLM_ROUTE(bf16, 8, 512); else if (tok == 4) PLLM_ROUTE(bf16, 4, 256); else PLLM_ROUTE(bf16, 1, kRouteThreads); }
 #undef PLLM_ROUTE
@@ -264,7 +279,8 @@ constexpr int kMoeCols = 64, kMoeK = 32;
 template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_expert_gemm_kernel(const T* __restrict__ rows_in, int ld_in, const T* __restrict__ w,
                                                               const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
-                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act,
+                                                              const float* __restrict__ pair_scale) {
   __shared__ float a_s[kMoeTileRows][kMoeK + 1];
   __shared__ float w_s[(GATED ? 2 : 1) * kMoeCols][kMoeK + 1];
   __shared__ int src[kMoeTileRows];
@@ -301,11 +317,12 @@ __global__ __launch_bounds__(256) void moe_expert_gemm_kernel(const T* __restric
     __syncthreads();
   }
   if (r >= nrows) return;
+  const float ps = (GATED && pair_scale) ? pair_scale[sorted_pair[row0 + r]] : 1.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int col = n0 + cg + 16 * j;
     if (col >= n_out) continue;
-    if (GATED) reinterpret_cast<T*>(out_)[(size_t)(row0 + r) * ld_out + col] = from_f32<T>(gate_activation(acc[j], act) * acc2[j]);
+    if (GATED) reinterpret_cast<T*>(out_)[(size_t)(row0 + r) * ld_out + col] = from_f32<T>(gate_activation(acc[j] * ps, act) * (acc2[j] * ps));
     else reinterpret_cast<float*>(out_)[(size_t)(row0 + r) * ld_out + col] = acc[j];
   }
 }
@@ -327,7 +344,8 @@ typedef __attribute__((ext_vector_type(4))) float moe_floatx4;
 template <bool GATED, int MT, int U>
 __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
                                                               const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
-                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act,
+                                                              const float* __restrict__ pair_scale) {
   constexpr int W = GATED ? 2 : 1;
   const int tile = blockIdx.x;
   const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
@@ -432,9 +450,10 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
       if (col >= n_out) continue;
       if (GATED) {
         bf16* o = reinterpret_cast<bf16*>(out_) + (size_t)(row0 + row) * ld_out + col;
+        const float ps = pair_scale ? pair_scale[sorted_pair[row0 + row]] : 1.f;      // a factor on the pair's input row
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[u][0][t][i], act) * acc[u][W - 1][t][i]);
+          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[u][0][t][i] * ps, act) * (acc[u][W - 1][t][i] * ps));
       } else {
         float* o = reinterpret_cast<float*>(out_) + (size_t)(row0 + row) * ld_out + col;
         if (col + 3 < n_out && (ld_out & 3) == 0) {
@@ -469,7 +488,8 @@ __device__ __forceinline__ void tile_barrier() {
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
                                                               const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
-                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act,
+                                                              const float* __restrict__ pair_scale) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[2][2][2][8 * 1024];   // [buffer][rows | weights][half of the k-step][8 blocks]
   const int tile = blockIdx.x;
   const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
@@ -570,13 +590,14 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
     const int row = wm * 64 + t * 16 + r;
     if (row >= nrows) continue;
     if (GATED) {
+      const float ps = pair_scale ? pair_scale[sorted_pair[row0 + row]] : 1.f;        // a factor on the pair's input row
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int col = n0 + wn * 32 + j * 16 + 4 * g;
         bf16* o = reinterpret_cast<bf16*>(out_) + (size_t)(row0 + row) * ld_out + col;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[j][t][i], act) * acc[j + 2][t][i]);
+          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[j][t][i] * ps, act) * (acc[j + 2][t][i] * ps));
       }
     } else {
 #pragma unroll
@@ -598,39 +619,42 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
 
 template <bool GATED>
 static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, int ld_in, const bf16* w, const int* tiles,
-                            const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, hipStream_t stream) {
+                            const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, const float* pair_scale,
+                            hipStream_t stream) {
   const int blocks = (n_out + 15) / 16;
   if (tile_rows >= kBigRows) {
     dim3 grid(max_tiles, GATED ? (n_out + 63) / 64 : (n_out + 127) / 128);
-    hipLaunchKernelGGL((moe_expert_tile_kernel<GATED>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+    hipLaunchKernelGGL((moe_expert_tile_kernel<GATED>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
   } else if (tile_rows >= 64) {
     constexpr int U = GATED ? 1 : 2;
     dim3 grid(max_tiles, (blocks + 4 * U - 1) / (4 * U));
-    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 4, U>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 4, U>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
   } else {
     dim3 grid(max_tiles, (blocks + 3) / 4);
-    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 1, 1>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 1, 1>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
   }
 }
 
+// pair_scale (gated product only, or null): a factor per pair, indexed like the ids, by which the pair's input row counts
+// as multiplied (it is applied to the gate's and the up product's float sums).
 // tile_rows: what moe_align was given.  Tiles of more than 16 rows are for the matrix-core kernel alone (bfloat16,
 // K and ld_in multiples of 8, 16-byte aligned operands); the plain kernel takes tiles of 16.
 PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int ld_in, const void* w, const int* tiles, int max_tiles,
                                   int tile_rows, const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act,
-                                  hipStream_t stream) {
+                                  const float* pair_scale, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || K <= 0 || top <= 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
   const bool matrix_cores = dtype == PLLM_BF16 && K % 8 == 0 && ld_in % 8 == 0 && ((uintptr_t)rows_in & 15) == 0 && ((uintptr_t)w & 15) == 0;
   if (tile_rows != kMoeTileRows && !(matrix_cores && (tile_rows == 64 || tile_rows == kMoeMaxTileRows))) return -2;
   if (matrix_cores) {
-    if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);
-    else launch_moe_mfma<false>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);
+    if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
+    else launch_moe_mfma<false>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
     PLLM_RETURN_LAST_ERROR();
   }
   dim3 grid(max_tiles, (n_out + kMoeCols - 1) / kMoeCols), block(256);
 #define PLLM_MOE(T, G)                                                                                                         \
   hipLaunchKernelGGL((moe_expert_gemm_kernel<T, G>), grid, block, 0, stream, (const T*)rows_in, ld_in, (const T*)w, tiles,    \
-                     sorted_pair, top, n_out, K, out, ld_out, act)
+                     sorted_pair, top, n_out, K, out, ld_out, act, pair_scale)
   if (dtype == PLLM_F32) { if (gated) PLLM_MOE(float, true); else PLLM_MOE(float, false); }
   else { if (gated) PLLM_MOE(bf16, true); else PLLM_MOE(bf16, false); }
 #undef PLLM_MOE
@@ -638,30 +662,41 @@ PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t, :] = sum_k weights[t, k] * (row_of_pair[t, k] >= 0 ? expert_out[row_of_pair[t, k], :] : h[t, :]), in the order of k.
+// out[t, :] = sum_k weights[t, k] * (row_of_pair[t, k] >= 0 ? expert_out[row_of_pair[t, k], :] : h[t, :]), in the order of k;
+// weights_inside: the experts' rows count once (their weight went into their input), only a pass-through row takes its weight.
+// shared (float [tokens, width], or null): + shared[t, :] * (shared_gate ? sigmoid(shared_gate[t * gate_ld]) : 1), a feed-forward
+// that every token passes, with one gate per token.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ expert_out, const T* __restrict__ h, int ld_h,
                                                           const int* __restrict__ row_of_pair, const float* __restrict__ weights,
+                                                          int weights_inside, const float* __restrict__ shared,
+                                                          const float* __restrict__ shared_gate, int gate_ld,
                                                           int top, int width, float* __restrict__ out) {
   const int t = blockIdx.x;
+  const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * gate_ld])) : 1.f) : 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
       const int row = row_of_pair[(size_t)t * top + k];
       const float v = row >= 0 ? expert_out[(size_t)row * width + i] : to_f32(h[(size_t)t * ld_h + i]);
-      acc = fmaf(weights[(size_t)t * top + k], v, acc);
+      if (weights_inside && row >= 0) acc += v;
+      else acc = fmaf(weights[(size_t)t * top + k], v, acc);
     }
+    if (shared) acc = fmaf(sg, shared[(size_t)t * width + i], acc);
     out[(size_t)t * width + i] = acc;
   }
 }
 
 PLLM_API int pllm_moe_combine(int dtype, const float* expert_out, const void* h, int ld_h, const int* row_of_pair, const float* weights,
+                              int weights_inside, const float* shared, const float* shared_gate, int gate_ld,
                               int num_tokens, int top, int width, float* out, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   dim3 grid(num_tokens), block(256);
   if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, expert_out, (const float*)h, ld_h, row_of_pair, weights, top, width, out);
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, expert_out, (const float*)h, ld_h, row_of_pair, weights,
+                       weights_inside, shared, shared_gate, gate_ld, top, width, out);
   else
-    hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, block, 0, stream, expert_out, (const bf16*)h, ld_h, row_of_pair, weights, top, width, out);
+    hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, block, 0, stream, expert_out, (const bf16*)h, ld_h, row_of_pair, weights,
+                       weights_inside, shared, shared_gate, gate_ld, top, width, out);
   PLLM_RETURN_LAST_ERROR();
 }

@@ -1245,7 +1245,7 @@ def recurrence_chunk(max_q_len: int, num_tokens: int) -> int:
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, state_offset: int,
                       state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
                       vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None, max_q_len: int = 0,
-                      step_sizes: tuple | None = None) -> torch.Tensor:
+                      step_sizes: tuple | None = None, normaliser: bool = False) -> torch.Tensor:
     """Per head:  S_t = decay_t S_(t-1) + k_t (vscale_t v_t)^T,   y_t = S_t^T q_t + skip v_t,   S [N, P] float32 at
     ``state[slot, state_offset + head * N * P :]``; a sequence with seq_starts == 0 starts from S = 0.
 
@@ -1254,6 +1254,8 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     per head for all tokens), vscale float32 [T, heads] or None, skip float32 [heads] or None.  Returns y float32 [T, heads * P].
     ``step_sizes`` = (raw [T, heads] view with unit inner stride, bias float32 [heads], a_log float32 [heads]) in place of
     ``decay`` (None) and ``vscale``: the kernel makes vscale_t = softplus(raw_t + bias) and decay_t = exp(-exp(a_log) vscale_t) itself.
+    ``normaliser``: S has one more column, P + 1, whose value is 1 at every token (it holds n_t = decay_t n_(t-1) + vscale_t k_t);
+    the state then takes heads * N * (P + 1) floats and y is [T, heads * (P + 1)] with n_t . q_t in every head's last column.
     ``max_q_len``: a bound on the tokens of one sequence in this step (0: unknown); from ``RECURRENCE_CHUNKS_FROM`` on the
     sequences are cut into chunks that run side by side (a chunk's own contribution from a zero state, the states carried
     from chunk to chunk, the outputs from each chunk's true starting state), which rounds differently than token by token."""
@@ -1262,7 +1264,8 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
           and q.stride(1) == q.shape[2], "recurrence q, k: [T, key_heads, N] views of one layout with the heads side by side")
     _need(v.dim() == 3 and v.stride(2) == 1 and v.stride(1) == v.shape[2] and v.shape[0] == q.shape[0], "recurrence v: [T, heads, P], heads side by side")
     T, KH, N = q.shape
-    H, P = v.shape[1], v.shape[2]
+    H, v_cols = v.shape[1], v.shape[2]
+    P = v_cols + 1 if normaliser else v_cols
     _need(H % KH == 0 and 1 <= N <= 1024, f"{H} heads over {KH} key heads, N = {N} (at most 1024)")
     raw = raw_bias = a_log = None
     if step_sizes is not None:
@@ -1286,13 +1289,13 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
            c_void_p, c_int, c_int, c_void_p, c_void_p,
            c_void_p, c_long, c_void_p, c_void_p,
-           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     _check(_fn("recurrent.hip", "pllm_linear_recurrence", signature=sig)(
         _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay),
         H if decay is not None and decay.dim() == 2 else 0, _ptr(vscale), _ptr(skip),
         _ptr(raw), dtype_code(raw.dtype) if raw is not None else 0, raw.stride(0) if raw is not None else 0, _ptr(raw_bias), _ptr(a_log),
         state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
-        _ptr(out), num_seqs, H, KH, N, P, chunk, max_chunks, _ptr(ws_state), _ptr(ws_decay), _stream()), "linear_recurrence")
+        _ptr(out), num_seqs, H, KH, N, P, v_cols, chunk, max_chunks, _ptr(ws_state), _ptr(ws_decay), _stream()), "linear_recurrence")
     return out
 
 
@@ -1314,41 +1317,101 @@ def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor |
     return out
 
 
+def mlstm_gates(raw_i: torch.Tensor, raw_f: torch.Tensor, bias_i: torch.Tensor | None, bias_f: torch.Tensor | None, cap: float,
+                state: torch.Tensor, m_at: int, state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor,
+                num_seqs: int) -> tuple:
+    """Log-domain gates of a matrix memory under a running maximum, per sequence and head, in float:
+    i = cap tanh((raw_i + bias_i) / cap), f = logsigmoid(cap tanh((raw_f + bias_f) / cap)) (cap 0: no cap),
+    m_t = max(f_t + m_(t-1), i_t) with m = 0 in front of a sequence's first token (``seq_starts`` == 0) and else what
+    ``state[slot, m_at + head]`` holds, where the last m is left.  Returns (decay, take, m), float32 [T, heads]:
+    exp(f_t + m_(t-1) - m_t), exp(i_t - m_t), m_t.  raw_i, raw_f: [T, heads] views of one type and row stride."""
+    _on_gpu(raw_i, raw_f, bias_i, bias_f, state, state_slots, seq_starts, cu_seqlens)
+    _need(raw_i.dim() == 2 and raw_i.shape == raw_f.shape and raw_i.stride() == raw_f.stride() and raw_i.stride(1) == 1
+          and raw_i.dtype == raw_f.dtype, "mlstm_gates: raw_i and raw_f are [T, heads] views of one layout")
+    T, H = raw_i.shape
+    for t in (bias_i, bias_f):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()), f"gate biases: float32 [{H}]")
+    _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
+    _need(0 <= m_at and m_at + H <= state.shape[1], "the running maxima do not fit the state slot")
+    decay, take, m = (torch.empty((T, H), dtype=torch.float32, device=raw_i.device) for _ in range(3))
+    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p,
+           c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_mlstm_gates", signature=sig)(
+        _ptr(raw_i), _ptr(raw_f), dtype_code(raw_i.dtype), raw_i.stride(0), _ptr(bias_i), _ptr(bias_f), c_float(cap), _ptr(state),
+        state.stride(0), m_at, _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens), _ptr(decay), _ptr(take), _ptr(m), num_seqs, H,
+        _stream()), "mlstm_gates")
+    return decay, take, m
+
+
+def mlstm_output(y: torch.Tensor, m: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor | None, heads: int, P: int, qscale: float,
+                 eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Behind ``linear_recurrence(..., normaliser=True)``: y float32 [T, heads * (P + 1)], m float32 [T, heads], gate
+    [T, heads * P] (a view, unit inner stride).  Per head o = y[:P] qscale / (max(|y[P] qscale|, exp(-m)) + 1e-6), then
+    o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate), as ``out_dtype`` [T, heads * P]."""
+    _on_gpu(y, m, gate, weight)
+    T = y.shape[0]
+    _need(y.dtype == torch.float32 and y.shape == (T, heads * (P + 1)) and y.is_contiguous(), f"mlstm_output y: float32 [T, {heads * (P + 1)}]")
+    _need(m.dtype == torch.float32 and m.shape == (T, heads) and m.is_contiguous(), f"m: float32 [{T}, {heads}]")
+    _need(gate.shape == (T, heads * P) and gate.stride(1) == 1, f"gate: [{T}, {heads * P}] with unit inner stride")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (heads * P,) and weight.is_contiguous()), f"weight: float32 [{heads * P}]")
+    out = torch.empty((T, heads * P), dtype=out_dtype, device=y.device)
+    sig = [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_mlstm_output", signature=sig)(
+        dtype_code(out_dtype), _ptr(y), _ptr(m), _ptr(gate), dtype_code(gate.dtype), gate.stride(0), _ptr(weight), _ptr(out), T, heads, P,
+        c_float(qscale), c_float(eps), _stream()), "mlstm_output")
+    return out
+
+
 # ------------------------------------------------------------------------------------------- attention over a latent
 MAX_LATENT_RANK, MAX_LATENT_ROT = 1024, 256
 
 
-def latent_prepare(rows: torch.Tensor, down_at: int, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor,
+def latent_prepare(rows: torch.Tensor, down_at: int, positions: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None, norm_weight: torch.Tensor,
                    eps: float, slots: torch.Tensor | None, k_pages: torch.Tensor, v_pages: torch.Tensor | None, q_out: torch.Tensor,
-                   heads: int, plain: int, rot: int, rank: int, interleaved: bool) -> None:
+                   heads: int, plain: int, rot: int, rank: int, interleaved: bool, q_latent: tuple | None = None) -> torch.Tensor | None:
     """From ``rows`` [T, heads x (plain | rot) | rank | rot] (the down-projection at column ``down_at``): the latent
     c = rms_norm(rows[down_at : down_at + rank]) * norm_weight and the key part behind it, turned by the tables' angles at
     ``positions``, go to the token's slot of ``k_pages`` [pages, 1, block, width] as the row [c | key part | 0], and c
     also to ``v_pages`` [pages, 1, width, block] (transposed inside the page) when given; no write for slot -1 or when
     ``slots`` is None.  Every head's rotated rot part goes to ``q_out`` [T, heads, width] at columns rank .. rank + rot,
-    zeros behind it (columns 0 .. rank are left alone: the query's latent-space part belongs there)."""
+    zeros behind it (columns 0 .. rank are left alone: the query's latent-space part belongs there).  ``rot`` 0: a latent
+    without a rotated part (no tables then; the rows need not hold the queries).  ``rows`` are of the pages' type or float32
+    (the sums of the product that made them).  ``q_latent`` = (column, q_rank, weight float32 [q_rank]): the rows also hold
+    a latent of the queries at that column; its RMS norm (the same eps) times the weight is returned in the pages' type,
+    [T, q_rank], the operand of the product that expands it into the heads' queries."""
     _on_gpu(rows, positions, cos, sin, norm_weight, slots, k_pages, v_pages, q_out)
-    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= down_at + rank + rot and down_at >= heads * (plain + rot),
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= down_at + rank + rot and (rot == 0 or down_at >= heads * (plain + rot)),
           "latent_prepare rows: [T, heads * (plain + rot) + rank + rot]")
+    _need(rows.dtype in (k_pages.dtype, torch.float32), "latent_prepare rows: of the pages' type, or float32")
     T = rows.shape[0]
-    _need(rot > 0 and rot % 2 == 0 and rank > 0, f"rot {rot} (even), rank {rank}")
+    _need(rot >= 0 and rot % 2 == 0 and rank > 0, f"rot {rot} (even), rank {rank}")
     _need(positions.dtype == torch.int32 and positions.numel() == T and positions.is_contiguous(), "positions: int32 [T]")
-    for t in (cos, sin):
-        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"rotary tables: float32 [positions, {rot // 2}]")
+    for t in (cos, sin) if rot else ():
+        _need(t is not None and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(),
+              f"rotary tables: float32 [positions, {rot // 2}]")
     _need(norm_weight.dtype == torch.float32 and norm_weight.shape == (rank,) and norm_weight.is_contiguous(), f"latent norm weight: float32 [{rank}]")
     _need(slots is None or (slots.dtype == torch.int32 and slots.numel() == T and slots.is_contiguous()), "slots: int32 [T]")
-    _need(k_pages.dim() == 4 and k_pages.shape[1] == 1 and k_pages.is_contiguous() and k_pages.dtype == rows.dtype, "k_pages: [pages, 1, block, width]")
+    _need(k_pages.dim() == 4 and k_pages.shape[1] == 1 and k_pages.is_contiguous(), "k_pages: [pages, 1, block, width]")
     pages, _, bs, width = k_pages.shape
     _need(width >= rank + rot, f"pages of width {width} for a latent of {rank} + {rot}")
-    _need(v_pages is None or (v_pages.shape == (pages, 1, width, bs) and v_pages.is_contiguous() and v_pages.dtype == rows.dtype),
+    _need(v_pages is None or (v_pages.shape == (pages, 1, width, bs) and v_pages.is_contiguous() and v_pages.dtype == k_pages.dtype),
           f"v_pages: [{pages}, 1, {width}, {bs}]")
-    _need(q_out.shape == (T, heads, width) and q_out.is_contiguous() and q_out.dtype == rows.dtype, f"q_out: contiguous [{T}, {heads}, {width}]")
-    sig = [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+    _need(q_out.shape == (T, heads, width) and q_out.is_contiguous() and q_out.dtype == k_pages.dtype, f"q_out: contiguous [{T}, {heads}, {width}]")
+    q_at = q_rank = 0
+    q_w = cq = None
+    if q_latent is not None:
+        q_at, q_rank, q_w = q_latent
+        _on_gpu(q_w)
+        _need(q_rank > 0 and 0 <= q_at and q_at + q_rank <= rows.shape[1] and q_w.dtype == torch.float32 and q_w.shape == (q_rank,) and q_w.is_contiguous(),
+              f"the queries' latent: {q_rank} columns at {q_at} with a float32 weight")
+        cq = torch.empty((T, q_rank), dtype=k_pages.dtype, device=rows.device)
+    sig = [c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     _check(_fn("latent_attention.hip", "pllm_latent_prepare", signature=sig)(
-        dtype_code(rows.dtype), _ptr(rows), rows.stride(0), down_at, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(norm_weight), c_float(eps),
-        _ptr(slots), _ptr(k_pages), _ptr(v_pages), _ptr(q_out), T, heads, plain, rot, rank, width, bs, 1 if interleaved else 0, _stream()),
-        "latent_prepare")
+        dtype_code(k_pages.dtype), dtype_code(rows.dtype), _ptr(rows), rows.stride(0), down_at, _ptr(positions), _ptr(cos) if rot else None, _ptr(sin) if rot else None, _ptr(norm_weight), c_float(eps),
+        _ptr(slots), _ptr(k_pages), _ptr(v_pages), _ptr(q_out), T, heads, plain, rot, rank, width, bs, 1 if interleaved else 0,
+        q_at, q_rank, _ptr(q_w), _ptr(cq), _stream()), "latent_prepare")
+    return cq
 
 
 def latent_attention(q: torch.Tensor, rank: int, rot: int, k_pages: torch.Tensor, block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor,
@@ -1459,6 +1522,37 @@ def place_rows(x: torch.Tensor, out: torch.Tensor) -> None:
         dtype_code(out.dtype), _ptr(x), _ptr(out), out.stride(0), x.shape[0], x.shape[1], _stream()), "place_rows")
 
 
+def dynamic_tanh(stream: torch.Tensor, alpha: float, weight: torch.Tensor | None, bias: torch.Tensor | None, branch: torch.Tensor | None = None,
+                 row_index: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """Around a float32 residual stream [rows, hidden]: with ``branch`` (float32 rows like the stream) stream += branch in
+    place; then, when ``out_dtype`` is given, the rows tanh(alpha * stream) * weight + bias of the stream as it is now are
+    returned in that type (``row_index``, int32, picks rows when no branch is added)."""
+    _on_gpu(stream, weight, bias, branch, row_index)
+    _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
+    rows, H = stream.shape
+    if branch is not None:
+        _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous() and row_index is None,
+              "a branch is contiguous float32 rows like the stream, and no rows are picked then")
+    if row_index is not None:
+        _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index must be contiguous int32")
+        rows = row_index.numel()
+    out = None
+    if out_dtype is not None:
+        for t, what in ((weight, "weight"), (bias, "bias")):
+            _need(t is not None and t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"{what} must be float32 [{H}]")
+        out = torch.empty((rows, H), dtype=out_dtype, device=stream.device)
+    _check(_fn("float_stream.hip", "pllm_dyt", signature=[c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_long,
+                                                         c_int, c_int, c_void_p])(
+        dtype_code(out_dtype or torch.float32), _ptr(branch), _ptr(stream), _ptr(row_index), c_float(alpha), _ptr(weight), _ptr(bias), _ptr(out),
+        H, rows, H, _stream()), "dynamic_tanh")
+    return out
+
+
+def stream_add(stream: torch.Tensor, branch: torch.Tensor) -> None:
+    """stream += branch in place, both contiguous float32 [rows, hidden] (a residual sum that nobody norms in the same kernel)."""
+    dynamic_tanh(stream, 0.0, None, None, branch)
+
+
 # ------------------------------------------------------------------------------------------- attention with normed queries and keys
 MAX_PREPARED_HEAD = 256
 
@@ -1466,12 +1560,13 @@ MAX_PREPARED_HEAD = 256
 def attn_prepare(proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Tensor | None, state: torch.Tensor | None,
                  state_slots, seq_starts, cu_seqlens, num_seqs: int, positions: torch.Tensor, cos: torch.Tensor | None,
                  sin: torch.Tensor | None, rot: int, interleaved: bool, eps: float, heads: int, kv_heads: int, d: int, dv: int, D: int,
-                 dtype: torch.dtype, slot_mapping: torch.Tensor | None, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None) -> torch.Tensor:
+                 dtype: torch.dtype, slot_mapping: torch.Tensor | None, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
+                 qk_norm: bool = True) -> torch.Tensor:
     """From the float32 sums ``proj`` [T, >= channels] of a q/k/v product (channels = heads d + kv_heads d + kv_heads dv):
     + ``bias``; a causal convolution over time per channel with ``conv_w`` float32 [channels, taps], whose inputs of
     earlier steps lie in ``state[slot]`` as [taps - 1, channels] and are left there for the next step; rotary encoding
     of the first ``rot`` elements of every q and k head; q and k heads divided by their root mean square (``eps``
-    inside the root); returns q as [T, heads * D] in ``dtype`` (heads padded with zeros to D) and writes k into
+    inside the root; not with ``qk_norm`` False); returns q as [T, heads * D] in ``dtype`` (heads padded with zeros to D) and writes k into
     ``k_pages`` [pages, kv_heads, block, D] and v into ``v_pages`` [pages, kv_heads, D, block] at ``slot_mapping``."""
     _on_gpu(proj, bias, conv_w, state, positions, cos, sin, slot_mapping, k_pages, v_pages)
     channels = (heads + kv_heads) * d + kv_heads * dv
@@ -1504,12 +1599,12 @@ def attn_prepare(proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Te
         _need(slot_mapping.dtype == torch.int32 and slot_mapping.numel() == T and slot_mapping.is_contiguous(), "slot_mapping: int32 [T]")
     q = torch.empty((T, heads * D), dtype=dtype, device=proj.device)
     sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-           c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
+           c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
     _check(_fn("attention_prepare.hip", "pllm_attn_prepare", signature=sig)(
         dtype_code(dtype), _ptr(proj), proj.stride(0), _ptr(bias), _ptr(conv_w), taps, _ptr(state) if taps > 1 else None,
         state.stride(0) if taps > 1 else 0, _ptr(state_slots) if taps > 1 else None, _ptr(seq_starts) if taps > 1 else None,
         _ptr(cu_seqlens) if taps > 1 else None, num_seqs, _ptr(positions), _ptr(cos) if rot else None, _ptr(sin) if rot else None, rot,
-        int(bool(interleaved)), c_float(eps), heads, kv_heads, d, dv, D, _ptr(q), _ptr(slot_mapping) if write else None,
+        int(bool(interleaved)), c_float(eps), int(bool(qk_norm)), heads, kv_heads, d, dv, D, _ptr(q), _ptr(slot_mapping) if write else None,
         _ptr(k_pages) if write else None, _ptr(v_pages) if write else None, bs, T, _stream()), "attn_prepare")
     return q
 
@@ -1535,25 +1630,34 @@ MOE_MAX_TILE_ROWS = 128
 MOE_MAX_EXPERTS = 1024
 
 
-def moe_route(h: torch.Tensor, router_w: torch.Tensor, correction: torch.Tensor | None, groups: int, keep: int, top: int) -> tuple:
-    """(ids int32 [T, top], weights float32 [T, top]): router outputs h router_w^T in float, softmax over all of them,
-    the ``top`` largest of score + correction among the experts of the ``keep`` best of ``groups`` groups of neighbours
-    (a group's mark: its largest corrected score), weights = the chosen experts' scores."""
+MOE_SCORINGS = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_route(h: torch.Tensor, router_w: torch.Tensor, correction: torch.Tensor | None, groups: int, keep: int, top: int,
+              scoring: str = "softmax", extra: int = 0) -> tuple:
+    """(ids int32 [T, top], weights float32 [T, top]): router outputs h router_w^T in float, scores by a softmax over all of
+    them or (``scoring`` "sigmoid") a sigmoid of each, the ``top`` largest of score + correction among the experts of the
+    ``keep`` best of ``groups`` groups of neighbours (a group's mark: its largest corrected score), weights = the chosen
+    experts' scores.  The last ``extra`` rows of ``router_w`` are no experts: their outputs come back as they are, as a
+    third result float32 [T, extra] (further products of the same rows that ride along)."""
     _on_gpu(h, router_w, correction)
     _need(h.dim() == 2 and h.stride(1) == 1, "moe_route rows: [T, width] with unit inner stride")
     T, W = h.shape
-    n = router_w.shape[0]
-    _need(router_w.dtype == torch.float32 and router_w.shape == (n, W) and router_w.is_contiguous(), f"router: float32 [n, {W}]")
+    n_all = router_w.shape[0]
+    n = n_all - extra
+    _need(scoring in MOE_SCORINGS and 0 <= extra < n_all, f"scoring {scoring!r} (one of {sorted(MOE_SCORINGS)}), {extra} extra rows of {n_all}")
+    _need(router_w.dtype == torch.float32 and router_w.shape == (n_all, W) and router_w.is_contiguous(), f"router: float32 [n, {W}]")
     _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (n,) and correction.is_contiguous()), f"correction: float32 [{n}]")
     _need(groups > 0 and n % groups == 0 and 0 < keep <= groups and 0 < top <= (n // groups) * keep,
           f"{n} router outputs in {groups} groups, {keep} kept, {top} chosen")
     ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
-    _check(_fn("moe.hip", "pllm_moe_route", signature=[c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                                        c_void_p, c_void_p, c_void_p])(
-        dtype_code(h.dtype), _ptr(h), h.stride(0), _ptr(router_w), _ptr(correction), T, W, n, groups, keep, top, _ptr(ids), _ptr(weights),
-        _stream()), "moe_route")
-    return ids, weights
+    extras = torch.empty((T, extra), dtype=torch.float32, device=h.device) if extra else None
+    _check(_fn("moe.hip", "pllm_moe_route", signature=[c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                                        c_int, c_void_p, c_void_p, c_void_p, c_void_p])(
+        dtype_code(h.dtype), _ptr(h), h.stride(0), _ptr(router_w), _ptr(correction), T, W, n_all, extra, MOE_SCORINGS[scoring], groups, keep, top,
+        _ptr(ids), _ptr(weights), _ptr(extras), _stream()), "moe_route")
+    return (ids, weights, extras) if extra else (ids, weights)
 
 
 def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, *inner_sizes: int) -> int:
@@ -1587,11 +1691,13 @@ def moe_align(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -
 
 
 def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor, sorted_pair: torch.Tensor, top: int, gated: bool,
-                    activation: str = "silu", tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
+                    activation: str = "silu", tile_rows: int = MOE_TILE_ROWS, pair_scale: torch.Tensor | None = None) -> torch.Tensor:
     """The experts' products over the sorted pairs.  ``gated``: rows_in [T, K] are the tokens' rows, w [experts, 2 N, K]
     holds [gate; up] per expert, the result [pairs, N] in the rows' type is act(gate . a) * (up . a) for the pair's token.
-    Else rows_in [pairs, K] are rows in sorted order, w [experts, N, K], and the result is float32 [pairs, N]."""
-    _on_gpu(rows_in, w, tiles, sorted_pair)
+    Else rows_in [pairs, K] are rows in sorted order, w [experts, N, K], and the result is float32 [pairs, N].
+    ``pair_scale`` (gated only; float32, one number per pair in the order of the ids): the pair's input row counts as
+    multiplied by it (the factor goes onto the gate's and the up product's float sums)."""
+    _on_gpu(rows_in, w, tiles, sorted_pair, pair_scale)
     _need(rows_in.dim() == 2 and rows_in.stride(1) == 1 and w.dim() == 3 and w.is_contiguous() and w.dtype == rows_in.dtype
           and w.shape[2] == rows_in.shape[1], f"moe_expert_gemm shapes {tuple(rows_in.shape)} x {tuple(w.shape)}")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous(), "tiles: int32 [n, 3]")
@@ -1603,25 +1709,37 @@ def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor,
     N = w.shape[1] // 2 if gated else w.shape[1]
     _need(gated or rows_in.shape[0] == pairs, "the down product takes one row per pair")
     _need(not gated or (w.shape[1] % 2 == 0 and rows_in.shape[0] * top == pairs), "the gated product takes the tokens' rows")
+    _need(pair_scale is None or (gated and pair_scale.dtype == torch.float32 and pair_scale.numel() == pairs and pair_scale.is_contiguous()),
+          f"pair_scale: float32 [{pairs}], for the gated product")
     out = torch.empty((pairs, N), dtype=rows_in.dtype if gated else torch.float32, device=rows_in.device)
     _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
-                                                              c_void_p, c_int, c_int, c_void_p])(
+                                                              c_void_p, c_int, c_int, c_void_p, c_void_p])(
         dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], tile_rows, _ptr(sorted_pair), top, N, K,
-        _ptr(out), out.stride(0), activation_code(activation), _stream()), "moe_expert_gemm")
+        _ptr(out), out.stride(0), activation_code(activation), _ptr(pair_scale), _stream()), "moe_expert_gemm")
     return out
 
 
-def moe_combine(expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+def moe_combine(expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor, weights_inside: bool = False,
+                shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
     """float32 [T, width]: sum over a token's choices, in their order, of weight * (the pair's row of ``expert_out``
-    [pairs, width] float32, or the token's own row of ``h`` where row_of_pair is -1)."""
-    _on_gpu(expert_out, h, row_of_pair, weights)
+    [pairs, width] float32, or the token's own row of ``h`` where row_of_pair is -1).  ``weights_inside``: the experts' rows
+    count once (their weight went into their input; a pass-through row still takes its weight).  ``shared`` (float32
+    [T, width]) is added, times sigmoid(shared_gate[t]) when ``shared_gate`` (float32 [T] or [T, 1], any row stride) is given."""
+    _on_gpu(expert_out, h, row_of_pair, weights, shared, shared_gate)
     T, top = weights.shape
     W = h.shape[1]
     _need(expert_out.dtype == torch.float32 and expert_out.shape == (T * top, W) and expert_out.is_contiguous(), f"expert outputs: float32 [{T * top}, {W}]")
     _need(h.dim() == 2 and h.shape[0] == T and h.stride(1) == 1, "moe_combine rows: [T, width]")
     _need(row_of_pair.dtype == torch.int32 and row_of_pair.numel() == T * top and row_of_pair.is_contiguous(), "row_of_pair: int32 [T * top]")
     _need(weights.dtype == torch.float32 and weights.is_contiguous(), "weights: float32 [T, top]")
+    _need(shared is None or (shared.dtype == torch.float32 and shared.shape == (T, W) and shared.is_contiguous()), f"shared: float32 [{T}, {W}]")
+    gate_ld = 0
+    if shared_gate is not None:
+        _need(shared is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() == T, f"shared_gate: float32 [{T}]")
+        gate_ld = shared_gate.stride(0)
     out = torch.empty((T, W), dtype=torch.float32, device=h.device)
-    _check(_fn("moe.hip", "pllm_moe_combine", signature=[c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p])(
-        dtype_code(h.dtype), _ptr(expert_out), _ptr(h), h.stride(0), _ptr(row_of_pair), _ptr(weights), T, top, W, _ptr(out), _stream()), "moe_combine")
+    _check(_fn("moe.hip", "pllm_moe_combine", signature=[c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                                          c_int, c_int, c_int, c_void_p, c_void_p])(
+        dtype_code(h.dtype), _ptr(expert_out), _ptr(h), h.stride(0), _ptr(row_of_pair), _ptr(weights), int(bool(weights_inside)), _ptr(shared),
+        _ptr(shared_gate), gate_ld, T, top, W, _ptr(out), _stream()), "moe_combine")
     return out

@@ -8,7 +8,10 @@
 //                          in the state slot: the state-space scan (k = B, q = C, v = x, a = exp(-exp(A_log) dt), g = dt,
 //                          skip = D) and retention (a = the head's decay, g = 1, no skip) are both this recurrence;
 //   gated_group_norm       the gate and the root-mean-square norm over groups of channels behind a recurrence, in
-//                          either order.
+//                          either order;
+//   mlstm_gates            log-domain input and forget gates of a matrix memory under a running maximum: the decays and
+//                          input factors that make it the linear recurrence above;
+//   mlstm_output           behind that recurrence: the division by the normaliser, the norm per head, the gate.
 //
 // A batch is token-major without padding: sequence s owns rows cu_seqlens[s] .. cu_seqlens[s + 1] - 1, its state
 // sits in slot state_slots[s], and seq_starts[s] == 0 says that it starts now, from a zero state, whatever the slot
@@ -212,6 +215,8 @@ struct RecurrenceArgs {
   long slot_stride;
   int qk_dtype, qk_stride, v_dtype, v_stride, decay_stride;
   int heads, key_heads, N, P, pblocks;
+  int v_cols;                          // columns of a head in v's rows: P, or P - 1 when the last column of S takes the value 1
+                                       // at every token (it then holds sum of decayed k_t g_t: a normaliser beside the memory)
 };
 
 // One workgroup per (sequence or chunk, head, block of 64 value channels); lane = value channel, so a token's update
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
     f.k = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
     f.q = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
-    f.x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
+    f.x = p < a.v_cols ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.v_cols + p) : (p_ok ? 1.f : 0.f);
     if (a.raw) {
       f.a = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head);
       f.g = 0.f;
@@ -380,6 +385,8 @@ static void launch_recurrence(const RecurrenceArgs& a, const ChunkArgs& ca, dim3
   else hipLaunchKernelGGL((linear_recurrence_kernel<64, 256, MODE>), grid, block, 0, stream, a, ca);
 }
 
+// v_cols: P, or P - 1 for a recurrence with a normaliser (v holds P - 1 columns per head; column P - 1 of S and of the output
+// belongs to the constant value 1).
 // chunk == 0: every sequence token by token in one workgroup per (head, block of channels).  chunk > 0: the three passes
 // over chunks of that many tokens; ws_state holds max_chunks * heads * N * P floats and ws_decay max_chunks * heads, with
 // max_chunks >= sum over the sequences of ceil(q_len / chunk) (total tokens / chunk + num_seqs is enough).
@@ -388,9 +395,9 @@ PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, 
                                     const void* raw, int raw_dtype, int raw_stride, const float* raw_bias, const float* a_log,
                                     float* state, long slot_stride, const int* state_slots, const int* seq_starts,
                                     const int* cu_seqlens, float* out, int num_seqs, int heads, int key_heads, int N, int P,
-                                    int chunk, int max_chunks, float* ws_state, float* ws_decay, hipStream_t stream) {
+                                    int v_cols, int chunk, int max_chunks, float* ws_state, float* ws_decay, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
-  if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0) return -2;
+  if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0 || (v_cols != P && v_cols != P - 1)) return -2;
   if ((raw && (!raw_bias || !a_log)) || (!raw && !decay)) return -2;
   if (chunk < 0 || (chunk > 0 && (max_chunks <= 0 || max_chunks > 65535 || !ws_state || !ws_decay)) || num_seqs > 65535) return -2;
   RecurrenceArgs a;
@@ -398,7 +405,7 @@ PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, 
   a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
   a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
   a.raw = raw; a.raw_dtype = raw_dtype; a.raw_stride = raw_stride; a.raw_bias = raw_bias; a.a_log = a_log;
-  a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64;
+  a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64; a.v_cols = v_cols;
   ChunkArgs ca{ws_state, ws_decay, chunk, num_seqs};
   const int waves = (N + 63) / 64, need = (N + waves - 1) / waves;   // rows of S per wave
   if (chunk == 0) {
@@ -569,5 +576,109 @@ PLLM_API int pllm_gated_group_norm(int dtype, const float* y, const void* gate, 
       hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
                          inner, group, gate_first, eps);
   }
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gates of a matrix memory with exponential input gates (mLSTM), per sequence and head, all in float:
+//   i_t = cap tanh((raw_i + b_i) / cap),   f_t = log sigmoid(cap tanh((raw_f + b_f) / cap))         (log-domain gates)
+//   m_t = max(f_t + m_(t-1), i_t)          a running maximum; m = 0 in front of a sequence's first token
+//   decay[t, h] = exp(f_t + m_(t-1) - m_t),   take[t, h] = exp(i_t - m_t),   m_out[t, h] = m_t,
+// so that S_t = decay_t S_(t-1) + take_t k_t v_t^T is the memory divided by exp(m_t).  m of a sequence's last token of
+// this step stays in state[slot][m_at + h].
+// One wavefront per (head, sequence) walks the sequence's tokens in blocks of 64: a lane makes its token's gates, and the
+// maxima are a scan over the lanes of the maps m -> max(a + m, b) ((a, b) of later tokens after (a', b') of earlier
+// ones is (a' + a, max(b' + a, b))); a lane past the sequence's end holds the identity (0, -inf).
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(const void* __restrict__ raw_i, const void* __restrict__ raw_f, int raw_dtype,
+                                                         int raw_stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
+                                                         float cap, float* state, long slot_stride, int m_at,
+                                                         const int* __restrict__ state_slots, const int* __restrict__ seq_starts,
+                                                         const int* __restrict__ cu_seqlens, float* __restrict__ decay,
+                                                         float* __restrict__ take, float* __restrict__ m_out, int heads) {
+  const int lane = threadIdx.x, head = blockIdx.x, seq = blockIdx.y;
+  const int q_begin = cu_seqlens[seq], q_len = cu_seqlens[seq + 1] - q_begin;
+  if (q_len <= 0) return;
+  float* st = state + (size_t)state_slots[seq] * slot_stride + m_at + head;
+  float m_in = seq_starts[seq] > 0 ? *st : 0.f;
+  const float bi = bias_i ? bias_i[head] : 0.f, bf = bias_f ? bias_f[head] : 0.f;
+  for (int t0 = 0; t0 < q_len; t0 += 64) {
+    const int t = t0 + lane;
+    const bool ok = t < q_len;
+    const size_t row = (size_t)(q_begin + (ok ? t : q_len - 1));
+    float gi = load_as_f32(raw_i, raw_dtype, row * raw_stride + head) + bi;
+    float gf = load_as_f32(raw_f, raw_dtype, row * raw_stride + head) + bf;
+    if (cap > 0.f) {
+      gi = cap * tanhf(gi / cap);
+      gf = cap * tanhf(gf / cap);
+    }
+    gf = fminf(gf, 0.f) - log1pf(expf(-fabsf(gf)));
+    float a = ok ? gf : 0.f, b = ok ? gi : -INFINITY;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float a_p = __shfl_up(a, off, 64), b_p = __shfl_up(b, off, 64);
+      if (lane >= off) {
+        b = fmaxf(b_p + a, b);
+        a = a_p + a;
+      }
+    }
+    const float m_t = fmaxf(a + m_in, b);
+    float m_prev = __shfl_up(m_t, 1, 64);
+    if (lane == 0) m_prev = m_in;
+    if (ok) {
+      const size_t at = row * heads + head;
+      decay[at] = expf(gf + m_prev - m_t);
+      take[at] = expf(gi - m_t);
+      m_out[at] = m_t;
+    }
+    m_in = __shfl(m_t, 63, 64);
+  }
+  if (lane == 0) *st = m_in;
+}
+
+PLLM_API int pllm_mlstm_gates(const void* raw_i, const void* raw_f, int raw_dtype, int raw_stride, const float* bias_i,
+                              const float* bias_f, float cap, float* state, long slot_stride, int m_at, const int* state_slots,
+                              const int* seq_starts, const int* cu_seqlens, float* decay, float* take, float* m_out, int num_seqs,
+                              int heads, hipStream_t stream) {
+  if (num_seqs <= 0) return 0;
+  if (heads <= 0 || num_seqs > 65535 || !raw_i || !raw_f || !state) return -2;
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(heads, num_seqs), dim3(64), 0, stream, raw_i, raw_f, raw_dtype, raw_stride, bias_i, bias_f,
+                     cap, state, slot_stride, m_at, state_slots, seq_starts, cu_seqlens, decay, take, m_out, heads);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// Behind the recurrence of a matrix memory with a normaliser: y [T, heads, P + 1] float holds S_t^T q_t in its first P
+// columns and n_t . q_t in the last; m [T, heads] the running maxima.  Per token and head, in float:
+//   o = y[:P] qscale / (max(|y[P] qscale|, exp(-m)) + 1e-6);   u = o / sqrt(mean(o^2) + eps) * w[head, :] * sigmoid(gate[head, :]);
+// out [T, heads * P] in the type T.  One wavefront per (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void mlstm_output_kernel(const float* __restrict__ y, const float* __restrict__ m, const void* __restrict__ gate,
+                                                          int gate_dtype, int gate_stride, const float* __restrict__ w, T* __restrict__ out,
+                                                          int heads, int P, float qscale, float eps) {
+  const int lane = threadIdx.x, tok = blockIdx.x, head = blockIdx.y;
+  const float* row = y + ((size_t)tok * heads + head) * (P + 1);
+  const float den = fmaxf(fabsf(row[P] * qscale), expf(-m[(size_t)tok * heads + head])) + 1e-6f;
+  const float f = qscale / den;
+  float sq = 0.f;
+  for (int p = lane; p < P; p += 64) {
+    const float o = row[p] * f;
+    sq = fmaf(o, o, sq);
+  }
+  const float inv = 1.f / sqrtf(wave_sum(sq) / (float)P + eps);
+  for (int p = lane; p < P; p += 64) {
+    const size_t c = (size_t)head * P + p;
+    const float g = load_as_f32(gate, gate_dtype, (size_t)tok * gate_stride + c);
+    out[(size_t)tok * heads * P + c] = from_f32<T>(row[p] * f * inv * (w ? w[c] : 1.f) / (1.f + expf(-g)));
+  }
+}
+
+PLLM_API int pllm_mlstm_output(int out_dtype, const float* y, const float* m, const void* gate, int gate_dtype, int gate_stride,
+                               const float* w, void* out, int num_tokens, int heads, int P, float qscale, float eps, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || heads > 65535 || P <= 0) return -2;
+  dim3 grid(num_tokens, heads), block(64);
+  if (out_dtype == PLLM_F32)
+    hipLaunchKernelGGL(mlstm_output_kernel<float>, grid, block, 0, stream, y, m, gate, gate_dtype, gate_stride, w, (float*)out, heads, P, qscale, eps);
+  else
+    hipLaunchKernelGGL(mlstm_output_kernel<bf16>, grid, block, 0, stream, y, m, gate, gate_dtype, gate_stride, w, (bf16*)out, heads, P, qscale, eps);
   PLLM_RETURN_LAST_ERROR();
 }

@@ -156,3 +156,70 @@ class SandwichNormBlock(Block):
 
 
 register_block("sandwich_norm", SandwichNormBlock)
+
+
+class FloatPreNormBlock(Block):
+    """The pre-norm block over a residual stream kept in float:
+
+        x <- x + mixer(norm_a(x));   x <- x + feed_forward(norm_b(x))        (the second line only with a feed-forward)
+
+    The branches' last products leave float rows (``ctx.float_branch``); the kernel that adds them to the stream in place
+    also computes, from the sums it holds, the rows of the norm that reads the stream next: this block's second norm, or
+    the first norm of the layer that follows (``ctx.next_entry_norm``, set by the model), which travel beside the stream in
+    ``ctx.launch_cache``.  The stream itself is never rounded.  The norms are of a kind with ``sum_then(stream, branch)``
+    (a norm whose rows need nothing but the row's own elements, or that computes its statistics in that kernel).
+
+    params: ``feed_forward`` (False: the mixer alone; the specs then name no feed-forward roles) and the roles' prefixes in
+    tensor names."""
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "feed_forward_norm": "norm", "feed_forward": "feed_forward"}
+    _ROWS = "float_prenorm_rows"
+
+    def __init__(self, params: dict, env):
+        self.has_feed_forward = bool(params.get("feed_forward", True))
+        if not self.has_feed_forward:
+            self.ROLES = {r: f for r, f in self.ROLES.items() if not r.startswith("feed_forward")}
+        super().__init__({k: v for k, v in params.items() if k in self.ROLES and isinstance(v, str)}, env)
+        self.dtype = env.dtype
+
+    def build_parts(self, specs, env):
+        super().build_parts(specs, env)
+        for role, family in self.ROLES.items():
+            if family == "norm" and not hasattr(self.parts[role], "sum_then"):
+                raise ValueError(f"the norm {type(self.parts[role]).__name__} of role {role!r} cannot follow a sum in its kernel (no sum_then)")
+
+    def entry_norm(self):
+        return self.parts["mixer_norm"]
+
+    def _entry_rows(self, x, ctx):
+        """norm_a(x) in the compute type: what the kernel that last wrote x left for this norm, or computed now."""
+        norm = self.parts["mixer_norm"]
+        held = ctx.launch_cache.get(self._ROWS)
+        if held is not None and held[0] is x and held[1] is norm:
+            return held[2]
+        return norm.forward(x)
+
+    def forward(self, x, delta, ctx, cache, state):
+        p = self.parts
+        if delta is not None:
+            raise RuntimeError("a block over a float stream takes the stream with every sum done")
+        if x.dtype != torch.float32:
+            raise RuntimeError("this block keeps its residual stream in float32 (an embedding with float_stream)")
+        after = getattr(ctx, "next_entry_norm", None)
+        after = after if hasattr(after, "sum_then") else None
+        ctx.partial_sums_ok, ctx.float_branch = False, True
+        a = p["mixer"].forward(self._entry_rows(x, ctx), ctx, cache, state)
+        if self.has_feed_forward:
+            h = p["feed_forward_norm"].sum_then(x, a)
+            a = p["feed_forward"].forward(h, ctx)
+        if after is not None:
+            rows = after.sum_then(x, a)
+            ctx.launch_cache[self._ROWS] = (x, after, rows)
+        else:
+            from ..csrc import ops
+            ops.stream_add(x, a)                                # the sum alone: whoever reads the stream next norms for itself
+            ctx.launch_cache[self._ROWS] = None
+        ctx.float_branch = False
+        return x, None
+
+
+register_block("prenorm_float_stream", FloatPreNormBlock)

@@ -178,3 +178,53 @@ class LayerNorm(Norm):
 
 
 register_norm("layernorm", LayerNorm)
+
+
+class DynamicTanh(Norm):
+    """A norm that computes no mean and no variance: y = tanh(alpha x) * w + b element by element, with a stored scalar
+    alpha, in float whatever the compute type.  ``forward`` gives the rows of a stream (float or compute-type rows) in
+    the compute type; ``sum_then`` adds a branch's float rows to a float residual stream in place and gives this
+    norm's rows of the new stream from the same kernel (a pre-norm block over a float stream: the kernel that forms a
+    sum also norms it for whoever reads the stream next).
+
+    params: ``size`` (default: the model's width); ``weight_name`` / ``bias_name`` / ``alpha_name``: the tensors' own
+    names under the part's prefix (defaults "weight", "bias", "alpha"; "" is the prefix itself)."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.size = int(params.get("size", env.hidden_size))
+        self.weight_name = params.get("weight_name", "weight")
+        self.bias_name = params.get("bias_name", "bias")
+        self.alpha_name = params.get("alpha_name", "alpha")
+        self.dtype, self.device = env.dtype, env.device
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+        self.alpha: float | None = None
+
+    def weight_specs(self):
+        return {self.weight_name: WeightSpec((self.size,), role="vector", init="ones"),
+                self.bias_name: WeightSpec((self.size,), role="vector", init="normal"),
+                self.alpha_name: WeightSpec((), role="vector", init="ones")}
+
+    def assign(self, name, tensor):
+        if name == self.alpha_name:
+            self.alpha = float(tensor.to(torch.float32))        # a constant of the kernel from here on
+            return
+        t = tensor.to(device=self.device, dtype=torch.float32).contiguous()
+        if name == self.weight_name:
+            self.weight = t
+        elif name == self.bias_name:
+            self.bias = t
+        else:
+            raise KeyError(name)
+
+    def forward(self, x, row_index=None):
+        if x.dtype != torch.float32:
+            x = x.float()
+        return ops.dynamic_tanh(x, self.alpha, self.weight, self.bias, None, row_index, self.dtype)
+
+    def sum_then(self, stream: torch.Tensor, branch: torch.Tensor) -> torch.Tensor:
+        """stream += branch in place (float); returns this norm's rows of the new stream in the compute type."""
+        return ops.dynamic_tanh(stream, self.alpha, self.weight, self.bias, branch, None, self.dtype)
+
+
+register_norm("dynamic_tanh", DynamicTanh)

@@ -1,4 +1,5 @@
-"""Causal attention over the paged cache whose queries and keys are divided by their root mean square per head.
+"""Causal attention over the paged cache whose queries and keys are prepared in float between the input product and the
+pages: usually divided by their root mean square per head (``qk_norm``; a layer may switch that off and keep the rest).
 
 q, k, v (and one gate per head) from one product of the mixer's input -> optional biases -> optional short causal
 convolution over time on every channel of q, k and v (the last taps - 1 projected rows of a request are its state) ->
@@ -30,7 +31,8 @@ class NormedAttention(Mixer):
     """params: ``heads``, ``kv_heads``, ``key_dim``, ``value_dim``, ``scale``, ``eps`` (of the q/k norm), ``position`` (a
     rotary spec or None), ``mask`` ("full", "window" or "chunk") with ``mask_size``, ``conv`` (taps of the convolution
     over time; 0: none), ``bias`` (q, k, v and the output product have biases), ``sinks`` (a logit per head in the
-    softmax's sum), ``head_gate`` (a gate per head from the mixer's input).  Tensors (under the part's prefix): ``q``,
+    softmax's sum), ``head_gate`` (a gate per head from the mixer's input), ``qk_norm`` (default True; False: q and k go
+    to the scores as they are rotated), ``score_cap`` c > 0 (the scaled product x becomes c tanh(x / c); default none).  Tensors (under the part's prefix): ``q``,
     ``k``, ``v``, ``o``; ``q.b``, ``k.b``, ``v.b``, ``o.b``; ``q.conv``, ``k.conv``, ``v.conv`` [channels, taps];
     ``sink`` [heads]; ``g`` [heads, width]."""
     graph_capturable = True
@@ -45,6 +47,9 @@ class NormedAttention(Mixer):
         self.has_conv = int(params.get("conv") or 0) >= 1
         self.taps = max(1, int(params.get("conv") or 1))
         self.bias, self.has_sinks, self.head_gate = bool(params.get("bias")), bool(params.get("sinks")), bool(params.get("head_gate"))
+        self.qk_norm, self.score_cap = bool(params.get("qk_norm", True)), float(params.get("score_cap") or 0.0)
+        if self.score_cap < 0.0:
+            raise ValueError(f"a cap of the scores is positive (or 0 for none), got {self.score_cap}")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads are no multiple of {self.kv_heads} kv heads")
         if self.mask not in MASKS or (self.mask != "full") != (self.mask_size > 0):
@@ -95,7 +100,7 @@ class NormedAttention(Mixer):
             self.output_bias = w.pop("o.b")           # added by whoever norms the mixer's float output (the block's kernel)
         if self.has_conv:
             self.conv_w = torch.cat([w.pop(n) for n in ("q.conv", "k.conv", "v.conv")], dim=0).contiguous()
-        terms = ops.ScoreTerms(0.0, None, w.pop("sink") if self.has_sinks else None)
+        terms = ops.ScoreTerms(self.score_cap, None, w.pop("sink") if self.has_sinks else None)
         self.terms = terms if terms.any() else None
 
     # ---- what it keeps
@@ -124,7 +129,7 @@ class NormedAttention(Mixer):
         q = ops.attn_prepare(proj, self.b_in, self.conv_w, state, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
                              ctx.positions, pe.cos if pe is not None else None, pe.sin if pe is not None else None, self.rot,
                              bool(pe.interleaved) if pe is not None else False, self.eps, H, G, self.d, self.dv, D, self.dtype,
-                             view.slot_mapping, k_pages, v_pages)
+                             view.slot_mapping, k_pages, v_pages, qk_norm=self.qk_norm)
         o = ops.paged_attention(q, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k, H, G, D, self.scale,
                                 self.window, ctx, terms=self.terms)
         if self.head_gate or D != self.dv:

@@ -11,6 +11,12 @@ Both are the same recurrence per head, S_t = a_t S_(t-1) + k_t (g_t v_t)^T, y_t 
   N^(-1/2), a constant decay per head; behind it each head's output divided by its root mean square, times
   silu(gate), the output product.
 
+* ``mlstm`` (a matrix memory with exponential input gates): q, k, v, an output gate and two gate pre-activations per
+  head from one product; the log-domain gates i and f run under a running maximum m, which makes a_t =
+  exp(f_t + m_(t-1) - m_t) and g_t = exp(i_t - m_t); a normaliser n_t (the same recurrence with k alone) is one more
+  column of S; y_t is divided by max(|n_t . q_t|, exp(-m_t)), then by its root mean square per head, times a weight,
+  times the sigmoid of the output gate, the output product.
+
 What enters the recurrence (step sizes, decays, rotated keys and queries, the state) is float whatever the compute type;
 the products, the convolution and the activations run in the compute type.  A request's state is zero at its first
 token (``ctx.seq_starts == 0``), whatever its slot held before.
@@ -147,5 +153,63 @@ class RetentionMixer(_StatefulMixer):
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
 
+class MLstmMixer(_StatefulMixer):
+    """A matrix memory per head with exponential input gates and sigmoid forget gates, kept in the log domain:
+
+        i_t = c tanh((W_i h + b_i) / c),   f_t = log sigmoid(c tanh((W_f h + b_f) / c)),   m_t = max(f_t + m_(t-1), i_t),  m_0 = 0
+        S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t the same with k_t alone
+        o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6),   q = W_q h N^(-1/2)
+
+    then each head's o divided by its root mean square, times ``norm`` (a weight over all heads' channels), times
+    sigmoid(W_g h), the output product.  The state slot holds S with n as its last column [heads, N, P + 1] and behind
+    it m [heads]; gates, maxima, state and what follows the recurrence are float whatever the compute type (the input
+    product leaves float sums).
+
+    params: ``heads``, ``key_dim`` (N), ``head_dim`` (P), ``gate_cap`` (c; 0: none), ``eps``.  Tensors ``q``, ``k`` [heads
+    N, width], ``v``, ``g`` [heads P, width], ``i``, ``f`` [heads, width] with ``i.b``, ``f.b`` [heads], ``norm`` [heads P],
+    ``o`` [width, heads P]."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.heads, self.N, self.P = int(params["heads"]), int(params["key_dim"]), int(params["head_dim"])
+        self.cap, self.eps = float(params.get("gate_cap") or 0.0), float(params["eps"])
+        if self.cap < 0.0:
+            raise ValueError(f"a cap of the gates is positive (or 0 for none), got {self.cap}")
+        self.dtype, self.device = env.dtype, env.device
+        self.m_at = self.heads * self.N * (self.P + 1)              # the running maxima lie behind S in the slot
+        self._w: dict = {}
+        self.w_in = self.w_o = None
+
+    def weight_specs(self):
+        H, qk, vg = self.heads, self.heads * self.N, self.heads * self.P
+        return {"q": WeightSpec((qk, self.hidden)), "k": WeightSpec((qk, self.hidden)), "v": WeightSpec((vg, self.hidden)),
+                "g": WeightSpec((vg, self.hidden)), "i": WeightSpec((H, self.hidden)), "f": WeightSpec((H, self.hidden)),
+                "i.b": WeightSpec((H,), role="vector"), "f.b": WeightSpec((H,), role="vector"),
+                "norm": WeightSpec((vg,), role="vector", init="ones"), "o": WeightSpec((self.hidden, vg))}
+
+    def finalize(self):
+        self.w_in = Weight(torch.cat([self._w.pop(n) for n in ("q", "k", "v", "g", "i", "f")], dim=0).contiguous())
+        self.w_o = Weight(self._w.pop("o"))
+
+    def state_spec(self):
+        return StateSpec((self.m_at + self.heads,), torch.float32)
+
+    def forward(self, h, ctx, cache, state):
+        H, N, P, w = self.heads, self.N, self.P, self._w
+        rows = linear(h, self.w_in, out_dtype=torch.float32)
+        qk, vg = H * N, H * P
+        q = rows[:, :qk].unflatten(1, (H, N))
+        k = rows[:, qk:2 * qk].unflatten(1, (H, N))
+        v = rows[:, 2 * qk:2 * qk + vg].unflatten(1, (H, P))
+        gate = rows[:, 2 * qk + vg:2 * qk + 2 * vg]
+        raw_i, raw_f = rows[:, 2 * qk + 2 * vg:2 * qk + 2 * vg + H], rows[:, 2 * qk + 2 * vg + H:]
+        seqs = (ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs)
+        decay, take, m = ops.mlstm_gates(raw_i, raw_f, w["i.b"], w["f.b"], self.cap, state, self.m_at, *seqs)
+        y = ops.linear_recurrence(q, k, v, decay, state, 0, *seqs, vscale=take, max_q_len=ctx.max_q_len, normaliser=True)
+        u = ops.mlstm_output(y, m, gate, w["norm"], H, P, N ** -0.5, self.eps, self.dtype)
+        return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
+
+
 register_mixer("mamba2", Mamba2Mixer)
 register_mixer("retention", RetentionMixer)
+register_mixer("mlstm", MLstmMixer)

@@ -39,6 +39,9 @@ class RotaryEncoding(PositionEncoding):
         self.scaling = params.get("scaling")
         self.rotary_dim = int(params.get("rotary_dim") or self.head_dim)
         self.interleaved = bool(params.get("interleaved", False))
+        # True: every frequency theta^(-2i/r) is formed in double precision and rounded to float once (default: float
+        # arithmetic all the way, as the reference's code has it; the two differ in the last place of some frequencies)
+        self.exact_frequencies = bool(params.get("exact_frequencies", False))
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary encoding turns pairs of elements: the rotated width must be even and at most the head "
                              f"size {self.head_dim}, got {self.rotary_dim}")
@@ -53,6 +56,13 @@ class RotaryEncoding(PositionEncoding):
 
     def inverse_frequencies(self) -> torch.Tensor:
         d = self.rotary_dim
+        if self.exact_frequencies:
+            inv_freq = torch.tensor([self.theta ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64)
+            if self.scaling:
+                s = self.scaling
+                inv_freq = llama3_rescale(inv_freq, float(s["factor"]), float(s.get("low_freq_factor", 1.0)), float(s.get("high_freq_factor", 4.0)),
+                                          int(s.get("original_max_position_embeddings", 8192)))
+            return inv_freq.to(torch.float32)
         inv_freq = 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
         if self.scaling:
             s = self.scaling
