@@ -171,12 +171,14 @@ def mlstm_mixer(h, w, m, eps):
         M_t = max(f_t + M_(t-1), i_t),   S_t = exp(f_t + M_(t-1) - M_t) S_(t-1) + exp(i_t - M_t) k_t v_t^T,
     n_t the same sum with k_t alone, o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-M_t)) + 1e-6)."""
     T = h.shape[0]
-    H, d, dv, cap = int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m["gate_cap"])
+    H, d, dv, cap = int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m.get("gate_cap") or 0.0)
     q = product(h, w["q"]).view(T, H, d) * d ** -0.5
     k = product(h, w["k"]).view(T, H, d)
     v = product(h, w["v"]).view(T, H, dv)
-    gi = cap * torch.tanh(product(h, w["i"], w["i.b"]) / cap)
-    gf = log_sigmoid(cap * torch.tanh(product(h, w["f"], w["f.b"]) / cap))
+    gi, gf = product(h, w["i"], w["i.b"]), product(h, w["f"], w["f.b"])
+    if cap > 0.0:                                            # (a cap of 0 stands for no cap)
+        gi, gf = cap * torch.tanh(gi / cap), cap * torch.tanh(gf / cap)
+    gf = log_sigmoid(gf)
     S = h.new_zeros((H, d, dv))
     n = h.new_zeros((H, d))
     M = h.new_zeros((H,))
