@@ -148,6 +148,60 @@ def run_mutapel(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
     return out
 
 
+def nesezen_config(width: int, vocab: int, window: int = 1024) -> dict:
+    """Nesezen at sizes that resemble a real model's layers: three periods of [windowed attention + dense feed-forward,
+    matrix memory + routed experts, latent attention + dense feed-forward, windowed attention + routed experts].  Heads of
+    64 elements on one key head per eight, a window of ``window`` positions, capped scores and rescaled frequencies; a
+    memory of width / 256 heads with 128 key rows and 256 value columns each; sixteen attention heads of 128 elements
+    over a latent of 256 with queries through a latent of three quarters of the width; 8 experts as wide as the model of
+    which 2 are chosen beside a shared one of three quarters of the width (the work of the dense feed-forward of 2.75
+    times the width)."""
+    heads = width // 64
+    att = {"heads": heads, "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 64, "mask": {"size": window}, "scale": 0.125, "softcap": 50.0,
+           "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}}}
+    mem = {"heads": max(1, width // 256), "dim": 128, "vdim": 256, "gate_cap": 15.0}
+    lat = {"heads": 16, "dim": 128, "vdim": 128, "kv_rank": 256, "q_rank": 3 * width // 4, "scale": 128 ** -0.5}
+    dense = {"kind": "dense", "ff": 11 * width // 4}
+    moe = {"kind": "moe", "expert": {"ff": width}, "router": {"experts": 8, "top": 2}, "shared": {"ff": 3 * width // 4}}
+    period = [{"type": "attention", "mixer": att, "mlp": dense}, {"type": "mlstm", "mixer": mem, "mlp": moe},
+              {"type": "latent_attention", "mixer": lat, "mlp": dense}, {"type": "attention", "mixer": att, "mlp": moe}]
+    return {"architecture": "Nesezen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [dict(l) for _ in range(3) for l in period], "max_positions": 4096, "torch_dtype": "bfloat16"}
+
+
+def run_nesezen(dtype: str, context: int, steps: int, warmup: int, widths=(1024, 2048)) -> dict:
+    """Prefill (one prompt of 512 and of 2048 tokens in one step) and decode (1, 8 and 64 requests at ``context``) of
+    Nesezen beside the two closest decoders at the same width, twelve layers and vocabulary (random weights): Gudutar (a
+    float residual stream, recurrent layers with a state per request, latent attention) and the Llama decoder."""
+    import torch
+    out = {}
+    for width in widths:
+        models = {
+            "nesezen": nesezen_config(width, 32000),
+            "gudutar": gudutar_config(width, 3, 32000),
+            "llama": dict(TINYLLAMA, num_hidden_layers=12, hidden_size=width, num_attention_heads=width // 64,
+                          num_key_value_heads=max(1, width // 512), head_dim=64, intermediate_size=11 * width // 4, torch_dtype=dtype),
+        }
+        for name, cfg in models.items():
+            row = {}
+            with tempfile.TemporaryDirectory() as folder:
+                engine = make_engine(cfg, folder, dtype, 64, context)
+                for tokens in (512, PREFILL_TOKENS):
+                    t = time_prefill(engine, tokens, seed=100 + tokens, repeats=4)
+                    row[f"prefill_{tokens}_ms"] = round(t * 1e3, 3)
+                    row[f"prefill_{tokens}_tok_per_s"] = round(tokens / t, 1)
+                for batch in (1, 8, 64):
+                    sec, _ = time_decode(engine, batch, context, steps, warmup, seed=batch)
+                    row[f"decode_b{batch}_ms"] = round(sec * 1e3, 4)
+                    row[f"decode_b{batch}_tok_per_s"] = round(batch / sec, 1)
+                row["weights_millions"] = round(sum(_weights_of(engine.model)) / 1e6, 1)
+                del engine
+                torch.cuda.empty_cache()
+            out[f"{name}_w{width}"] = row
+            print(f"[bench] {name} width {width}: {row}", file=sys.stderr, flush=True)
+    return out
+
+
 def _weights_of(model):
     """Numbers of elements of the tensors the model declares (what a checkpoint of it holds)."""
     out = []
@@ -672,6 +726,8 @@ def main() -> int:
                     "latent-attention layers) at two widths beside the Llama decoder of the same width and depth, instead")
     ap.add_argument("--mutapel", action="store_true", help="prefill and decode of the Mutapel decoder (windowed and blocked attention with "
                     "normed queries and keys, routed experts) beside a Llama decoder of the same width and depth, and nothing else")
+    ap.add_argument("--nesezen", action="store_true", help="prefill and decode of the Nesezen decoder (windowed attention with capped scores, a "
+                    "matrix memory, latent attention, routed experts with a shared one) beside Gudutar and the Llama decoder at equal width and depth, and nothing else")
     ap.add_argument("--kernels", action="store_true", help="every kernel of a decode step and of a prompt step on its own, with its fraction")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -698,6 +754,11 @@ def main() -> int:
         print(json.dumps({"metric": "Mutapel beside the Llama decoder at equal width, layer runs, heads and vocabulary (random weights): prefill and decode",
                           "dtype": short, "context": args.context,
                           "models": run_mutapel(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
+        return 0
+    if args.nesezen:
+        print(json.dumps({"metric": "Nesezen beside Gudutar and the Llama decoder at equal width, depth and vocabulary (random weights): prefill and decode",
+                          "dtype": short, "context": args.context,
+                          "models": run_nesezen(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
         return 0
     if args.workload == "ragged64":
         print(json.dumps({"metric": f"output tokens/s, 64 ragged requests at once, prompts 64-2048 tokens, 256 generated each ({model_name}, random weights)",
