@@ -434,3 +434,49 @@ PLLM_API int pllm_dyt(int out_dtype, const float* branch, float* stream, const i
     hipLaunchKernelGGL(dyt_kernel<bf16>, grid, block, 0, stream_, branch, stream, row_index, alpha, w, b, (bf16*)rows, rows_stride, hidden, vec);
   PLLM_RETURN_LAST_ERROR();
 }
+
+// The same behind routed experts, whose weighted sum this kernel forms where it would have read the branch:
+//   branch[r] = sum_k (weights_inside && row >= 0 ? 1 : weights[r, k]) * (row >= 0 ? expert_out[row] : h[r]),  row = row_of_pair[r, k],
+//               in the order of k, + shared[r] * (shared_gate ? sigmoid(shared_gate[r * gate_ld]) : 1) when shared is given;
+//   stream[r] += branch[r];   rows[r] = T(tanh(alpha * stream[r]) * w + b) when rows is given.
+template <typename TO, typename TH>
+__global__ __launch_bounds__(256) void dyt_sum_kernel(const float* __restrict__ expert_out, const TH* __restrict__ h, long ld_h,
+                                                      const int* __restrict__ row_of_pair, const float* __restrict__ weights, int top,
+                                                      int weights_inside, const float* __restrict__ shared,
+                                                      const float* __restrict__ shared_gate, int gate_ld, float* stream, float alpha,
+                                                      const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ rows,
+                                                      long rows_stride, int hidden) {
+  const int r = blockIdx.x;
+  float* x = stream + (size_t)r * hidden;
+  TO* out = rows ? rows + (size_t)r * rows_stride : nullptr;
+  const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)r * gate_ld])) : 1.f) : 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = row_of_pair[(size_t)r * top + k];
+      const float v = row >= 0 ? expert_out[(size_t)row * hidden + i] : to_f32(h[(size_t)r * ld_h + i]);
+      if (weights_inside && row >= 0) acc += v;
+      else acc = fmaf(weights[(size_t)r * top + k], v, acc);
+    }
+    if (shared) acc = fmaf(sg, shared[(size_t)r * hidden + i], acc);
+    const float v = x[i] + acc;
+    x[i] = v;
+    if (out) out[i] = from_f32<TO>(fmaf(tanhf(alpha * v), w[i], b[i]));
+  }
+}
+
+PLLM_API int pllm_dyt_sum(int out_dtype, int h_dtype, const float* expert_out, const void* h, long ld_h, const int* row_of_pair,
+                          const float* weights, int top, int weights_inside, const float* shared, const float* shared_gate, int gate_ld,
+                          float* stream, float alpha, const float* w, const float* b, void* rows, long rows_stride, int num_rows,
+                          int hidden, hipStream_t stream_) {
+  if (num_rows <= 0) return 0;
+  if (top <= 0 || (rows && (!w || !b))) return -2;
+  dim3 grid(num_rows), block(hidden >= 1024 ? 256 : (hidden >= 128 ? 128 : 64));
+#define PLLM_DS(TO, TH)                                                                                                              \
+  hipLaunchKernelGGL((dyt_sum_kernel<TO, TH>), grid, block, 0, stream_, expert_out, (const TH*)h, ld_h, row_of_pair, weights, top,    \
+                     weights_inside, shared, shared_gate, gate_ld, stream, alpha, w, b, (TO*)rows, rows_stride, hidden)
+  if (out_dtype == PLLM_F32) { if (h_dtype == PLLM_F32) PLLM_DS(float, float); else PLLM_DS(float, bf16); }
+  else { if (h_dtype == PLLM_F32) PLLM_DS(bf16, float); else PLLM_DS(bf16, bf16); }
+#undef PLLM_DS
+  PLLM_RETURN_LAST_ERROR();
+}

@@ -1446,11 +1446,19 @@ class ChoiceSum:
     the pair's row of ``expert_out`` (float32 [pairs, width]) or, where ``row_of_pair`` is -1, the token's own row of
     ``h``.  ``rows()`` forms it (``moe_combine``); ``rms_sandwich`` takes it as a branch and forms it in its own kernel."""
 
-    def __init__(self, expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor):
+    def __init__(self, expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor,
+                 weights_inside: bool = False, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None):
         self.expert_out, self.h, self.row_of_pair, self.weights = expert_out, h, row_of_pair, weights
+        # (as ``moe_combine`` takes them: weights that went into the experts' inputs, a feed-forward that every token passes)
+        self.weights_inside, self.shared, self.shared_gate = bool(weights_inside), shared, shared_gate
+
+    @property
+    def plain(self) -> bool:
+        """Whether the sum is the weighted sum of the choices and nothing else."""
+        return not self.weights_inside and self.shared is None
 
     def rows(self) -> torch.Tensor:
-        return moe_combine(self.expert_out, self.h, self.row_of_pair, self.weights)
+        return moe_combine(self.expert_out, self.h, self.row_of_pair, self.weights, self.weights_inside, self.shared, self.shared_gate)
 
     def checked(self, rows: int, width: int):
         e, h, rp, wt = self.expert_out, self.h, self.row_of_pair, self.weights
@@ -1479,8 +1487,8 @@ def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: to
     for t, what in ((w_branch, "w_branch"), (w_next, "w_next"), (bias, "bias")):
         _need(t is None or (t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()), f"{what} must be float32 [{H}]")
     if isinstance(branch, ChoiceSum):
-        if H > SANDWICH_HELD_MAX:
-            branch = branch.rows()                          # (rows too long for the kernel that holds them in registers)
+        if H > SANDWICH_HELD_MAX or not branch.plain:
+            branch = branch.rows()                          # (rows too long for the kernel that holds them in registers, or a sum with further terms)
         else:
             _need(row_index is None and w_branch is not None, "a branch comes with its norm's weight, and no rows are picked")
             if out is None and out_dtype is not None:
@@ -1522,14 +1530,34 @@ def place_rows(x: torch.Tensor, out: torch.Tensor) -> None:
         dtype_code(out.dtype), _ptr(x), _ptr(out), out.stride(0), x.shape[0], x.shape[1], _stream()), "place_rows")
 
 
-def dynamic_tanh(stream: torch.Tensor, alpha: float, weight: torch.Tensor | None, bias: torch.Tensor | None, branch: torch.Tensor | None = None,
+def dynamic_tanh(stream: torch.Tensor, alpha: float, weight: torch.Tensor | None, bias: torch.Tensor | None, branch=None,
                  row_index: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
-    """Around a float32 residual stream [rows, hidden]: with ``branch`` (float32 rows like the stream) stream += branch in
-    place; then, when ``out_dtype`` is given, the rows tanh(alpha * stream) * weight + bias of the stream as it is now are
+    """Around a float32 residual stream [rows, hidden]: with ``branch`` (float32 rows like the stream, or a ``ChoiceSum``: a
+    weighted sum of experts' rows that the kernel forms itself) stream += branch in place; then, when ``out_dtype`` is given, the rows tanh(alpha * stream) * weight + bias of the stream as it is now are
     returned in that type (``row_index``, int32, picks rows when no branch is added)."""
-    _on_gpu(stream, weight, bias, branch, row_index)
+    _on_gpu(stream, weight, bias, None if isinstance(branch, ChoiceSum) else branch, row_index)
     _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
     rows, H = stream.shape
+    if isinstance(branch, ChoiceSum):
+        # the experts' weighted sum (with what rides on it) is formed by the kernel that adds it to the stream
+        _need(row_index is None, "no rows are picked where a branch is added")
+        e, h, rp, wt = branch.checked(rows, H)
+        shared, gate = branch.shared, branch.shared_gate
+        _on_gpu(shared, gate)
+        _need(shared is None or (shared.dtype == torch.float32 and shared.shape == (rows, H) and shared.is_contiguous()), f"shared: float32 [{rows}, {H}]")
+        _need(gate is None or (shared is not None and gate.dtype == torch.float32 and gate.numel() == rows), f"shared_gate: float32 [{rows}]")
+        out = None
+        if out_dtype is not None:
+            for t, what in ((weight, "weight"), (bias, "bias")):
+                _need(t is not None and t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"{what} must be float32 [{H}]")
+            out = torch.empty((rows, H), dtype=out_dtype, device=stream.device)
+        sig = [c_int, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p,
+               c_void_p, c_void_p, c_long, c_int, c_int, c_void_p]
+        _check(_fn("float_stream.hip", "pllm_dyt_sum", signature=sig)(
+            dtype_code(out_dtype or torch.float32), dtype_code(h.dtype), _ptr(e), _ptr(h), h.stride(0), _ptr(rp), _ptr(wt), wt.shape[1],
+            int(branch.weights_inside), _ptr(shared), _ptr(gate), gate.stride(0) if gate is not None else 0, _ptr(stream), c_float(alpha),
+            _ptr(weight), _ptr(bias), _ptr(out), H, rows, H, _stream()), "dynamic_tanh_sum")
+        return out
     if branch is not None:
         _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous() and row_index is None,
               "a branch is contiguous float32 rows like the stream, and no rows are picked then")
@@ -1548,8 +1576,9 @@ def dynamic_tanh(stream: torch.Tensor, alpha: float, weight: torch.Tensor | None
     return out
 
 
-def stream_add(stream: torch.Tensor, branch: torch.Tensor) -> None:
-    """stream += branch in place, both contiguous float32 [rows, hidden] (a residual sum that nobody norms in the same kernel)."""
+def stream_add(stream: torch.Tensor, branch) -> None:
+    """stream += branch in place: contiguous float32 [rows, hidden], the branch also a ``ChoiceSum`` (a residual sum that nobody
+    norms in the same kernel)."""
     dynamic_tanh(stream, 0.0, None, None, branch)
 
 

@@ -210,7 +210,9 @@ class FloatPreNormBlock(Block):
         a = p["mixer"].forward(self._entry_rows(x, ctx), ctx, cache, state)
         if self.has_feed_forward:
             h = p["feed_forward_norm"].sum_then(x, a)
+            ctx.branch_sum_ok = True      # a feed-forward may hand over a sum that the kernel behind it forms (``ops.ChoiceSum``)
             a = p["feed_forward"].forward(h, ctx)
+            ctx.branch_sum_ok = False
         if after is not None:
             rows = after.sum_then(x, a)
             ctx.launch_cache[self._ROWS] = (x, after, rows)

@@ -110,8 +110,9 @@ class RoutedExperts(FeedForward):
         if self.shared_inter:
             shared = linear(gated_linear(h, self.w_shared_gate_up, self.activation), self.w_shared_down, out_dtype=torch.float32)
             gate = routed[2] if self.shared_gate else None
-        if not inside and shared is None and getattr(ctx, "float_branch", False) and getattr(ctx, "branch_sum_ok", False):
-            return ops.ChoiceSum(out, h, row_of_pair, weights)      # whoever norms the branch forms the sum in its kernel
+        if getattr(ctx, "float_branch", False) and getattr(ctx, "branch_sum_ok", False):
+            # whoever takes the branch forms the sum in its kernel
+            return ops.ChoiceSum(out, h, row_of_pair, weights, inside, shared, gate)
         y = ops.moe_combine(out, h, row_of_pair, weights, inside, shared, gate)
         if getattr(ctx, "float_branch", False):
             return y
