@@ -465,12 +465,89 @@ __global__ __launch_bounds__(256) void dyt_sum_kernel(const float* __restrict__ 
   }
 }
 
+// The same with four elements per thread and load, the choices' rows and weights read once per workgroup into LDS and
+// the rows of four choices asked for before the first of them is added (hidden a multiple of 4, at most kSumTop choices,
+// rows on 16-byte boundaries): the loads of a step no longer wait for one another.
+constexpr int kSumTop = 64, kSumAhead = 4;
+
+template <typename TO, typename TH>
+__global__ __launch_bounds__(256) void dyt_sum_vec_kernel(const float* __restrict__ expert_out, const TH* __restrict__ h, long ld_h,
+                                                          const int* __restrict__ row_of_pair, const float* __restrict__ weights, int top,
+                                                          int weights_inside, const float* __restrict__ shared,
+                                                          const float* __restrict__ shared_gate, int gate_ld, float* stream, float alpha,
+                                                          const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ rows,
+                                                          long rows_stride, int hidden) {
+  __shared__ int row_s[kSumTop];
+  __shared__ float weight_s[kSumTop];
+  const int r = blockIdx.x;
+  if ((int)threadIdx.x < top) {
+    const int row = row_of_pair[(size_t)r * top + threadIdx.x];
+    row_s[threadIdx.x] = row;
+    weight_s[threadIdx.x] = (weights_inside && row >= 0) ? 1.f : weights[(size_t)r * top + threadIdx.x];
+  }
+  float* x = stream + (size_t)r * hidden;
+  TO* out = rows ? rows + (size_t)r * rows_stride : nullptr;
+  const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)r * gate_ld])) : 1.f) : 0.f;
+  __syncthreads();
+  for (int i = 4 * threadIdx.x; i < hidden; i += 4 * blockDim.x) {
+    const float4 x4 = *reinterpret_cast<const float4*>(x + i);
+    float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (shared) s4 = *reinterpret_cast<const float4*>(shared + (size_t)r * hidden + i);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k0 = 0; k0 < top; k0 += kSumAhead) {
+      float4 v[kSumAhead];
+#pragma unroll
+      for (int j = 0; j < kSumAhead; ++j) {
+        const int k = k0 + j < top ? k0 + j : top - 1;
+        const int row = row_s[k];
+        if (row >= 0) v[j] = *reinterpret_cast<const float4*>(expert_out + (size_t)row * hidden + i);
+        else v[j] = make_float4(to_f32(h[(size_t)r * ld_h + i]), to_f32(h[(size_t)r * ld_h + i + 1]), to_f32(h[(size_t)r * ld_h + i + 2]),
+                                to_f32(h[(size_t)r * ld_h + i + 3]));
+      }
+#pragma unroll
+      for (int j = 0; j < kSumAhead; ++j)
+        if (k0 + j < top) {
+          const float wt = weight_s[k0 + j];
+          if (weights_inside && row_s[k0 + j] >= 0) { acc.x += v[j].x; acc.y += v[j].y; acc.z += v[j].z; acc.w += v[j].w; }
+          else { acc.x = fmaf(wt, v[j].x, acc.x); acc.y = fmaf(wt, v[j].y, acc.y); acc.z = fmaf(wt, v[j].z, acc.z); acc.w = fmaf(wt, v[j].w, acc.w); }
+        }
+    }
+    if (shared) { acc.x = fmaf(sg, s4.x, acc.x); acc.y = fmaf(sg, s4.y, acc.y); acc.z = fmaf(sg, s4.z, acc.z); acc.w = fmaf(sg, s4.w, acc.w); }
+    const float4 v = make_float4(x4.x + acc.x, x4.y + acc.y, x4.z + acc.z, x4.w + acc.w);
+    *reinterpret_cast<float4*>(x + i) = v;
+    if (out) {
+      const float4 ww = *reinterpret_cast<const float4*>(w + i), bb = *reinterpret_cast<const float4*>(b + i);
+      Quad<TO> o;
+      o.v[0] = from_f32<TO>(fmaf(tanhf(alpha * v.x), ww.x, bb.x));
+      o.v[1] = from_f32<TO>(fmaf(tanhf(alpha * v.y), ww.y, bb.y));
+      o.v[2] = from_f32<TO>(fmaf(tanhf(alpha * v.z), ww.z, bb.z));
+      o.v[3] = from_f32<TO>(fmaf(tanhf(alpha * v.w), ww.w, bb.w));
+      *reinterpret_cast<Quad<TO>*>(out + i) = o;
+    }
+  }
+}
+
 PLLM_API int pllm_dyt_sum(int out_dtype, int h_dtype, const float* expert_out, const void* h, long ld_h, const int* row_of_pair,
                           const float* weights, int top, int weights_inside, const float* shared, const float* shared_gate, int gate_ld,
                           float* stream, float alpha, const float* w, const float* b, void* rows, long rows_stride, int num_rows,
                           int hidden, hipStream_t stream_) {
   if (num_rows <= 0) return 0;
   if (top <= 0 || (rows && (!w || !b))) return -2;
+  const size_t out_bytes = out_dtype == PLLM_F32 ? 4 : 2;
+  const bool vec = hidden % 4 == 0 && top <= kSumTop && ((uintptr_t)stream & 15) == 0 && ((uintptr_t)expert_out & 15) == 0 &&
+                   (!shared || ((uintptr_t)shared & 15) == 0) &&
+                   (!rows || (((uintptr_t)rows % (4 * out_bytes)) == 0 && rows_stride % 4 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)b & 15) == 0));
+  if (vec) {
+    const int threads = hidden >= 1024 ? 256 : (hidden / 4 + 63) / 64 * 64;
+    dim3 vgrid(num_rows), vblock(threads < 64 ? 64 : threads);
+#define PLLM_DSV(TO, TH)                                                                                                              \
+  hipLaunchKernelGGL((dyt_sum_vec_kernel<TO, TH>), vgrid, vblock, 0, stream_, expert_out, (const TH*)h, ld_h, row_of_pair, weights, top, \
+                     weights_inside, shared, shared_gate, gate_ld, stream, alpha, w, b, (TO*)rows, rows_stride, hidden)
+    if (out_dtype == PLLM_F32) { if (h_dtype == PLLM_F32) PLLM_DSV(float, float); else PLLM_DSV(float, bf16); }
+    else { if (h_dtype == PLLM_F32) PLLM_DSV(bf16, float); else PLLM_DSV(bf16, bf16); }
+#undef PLLM_DSV
+    PLLM_RETURN_LAST_ERROR();
+  }
   dim3 grid(num_rows), block(hidden >= 1024 ? 256 : (hidden >= 128 ? 128 : 64));
 #define PLLM_DS(TO, TH)                                                                                                              \
   hipLaunchKernelGGL((dyt_sum_kernel<TO, TH>), grid, block, 0, stream_, expert_out, (const TH*)h, ld_h, row_of_pair, weights, top,    \
