@@ -215,8 +215,9 @@ struct RecurrenceArgs {
   long slot_stride;
   int qk_dtype, qk_stride, v_dtype, v_stride, decay_stride;
   int heads, key_heads, N, P, pblocks;
-  int v_cols;                          // columns of a head in v's rows: P, or P - 1 when the last column of S takes the value 1
-                                       // at every token (it then holds sum of decayed k_t g_t: a normaliser beside the memory)
+  int ld;                              // elements of a row of S in the state and of a head in the output rows: P, or P + 1 when a
+                                       // normaliser n_t = a_t n_(t-1) + g_t k_t stands behind the P columns (n as the last column of
+                                       // S, n_t . q_t as the last element of the head's output)
 };
 
 // One workgroup per (sequence or chunk, head, block of 64 value channels); lane = value channel, so a token's update
@@ -256,6 +257,7 @@ __device__ __forceinline__ bool find_chunk(const int* __restrict__ cu_seqlens, i
 template <int NR, int MAX_THREADS, int MODE>
 __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(RecurrenceArgs a, ChunkArgs ca) {
   __shared__ float part[2][MAX_THREADS / 64][64];
+  __shared__ float part_n[2][MAX_THREADS / 64];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
   const int head = blockIdx.x / a.pblocks, pb = blockIdx.x % a.pblocks;
   const int p = pb * 64 + lane;
@@ -269,15 +271,20 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
   const int kh = head / (a.heads / a.key_heads);
   const int n0 = wv * NR;
   const bool carried = a.seq_starts[seq] > 0;
-  float* st = MODE == kWhole ? a.state + (size_t)a.state_slots[seq] * a.slot_stride + (size_t)head * a.N * a.P
-                             : ca.ws_state + ((size_t)blockIdx.y * a.heads + head) * a.N * a.P;
+  const int ld = a.ld;
+  float* st = MODE == kWhole ? a.state + (size_t)a.state_slots[seq] * a.slot_stride + (size_t)head * a.N * ld
+                             : ca.ws_state + ((size_t)blockIdx.y * a.heads + head) * a.N * ld;
+  const bool from_state = MODE != kChunkState && (MODE == kChunkOut || carried);
   float S[NR];
 #pragma unroll
-  for (int i = 0; i < NR; ++i)
-    S[i] = (MODE != kChunkState && (MODE == kChunkOut || carried) && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * a.P + p] : 0.f;
+  for (int i = 0; i < NR; ++i) S[i] = (from_state && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * ld + p] : 0.f;
   const float skip = a.skip ? a.skip[head] : 0.f;
   const float rate = a.raw ? expf(a.a_log[head]) : 0.f, raw_bias = a.raw ? a.raw_bias[head] : 0.f;
   const bool mine = lane < NR && n0 + lane < a.N;
+  // The normaliser, where there is one: lane l of wave w holds n[w * NR + l], the row whose k and q it fetches anyway, so its
+  // update is one multiply-add a token and n . q one sum over the wavefront; the head's first block of columns keeps it.
+  const bool with_n = ld > a.P && pb == 0;
+  float nl = (with_n && from_state && mine) ? st[(size_t)(n0 + lane) * ld + a.P] : 0.f;
   float decays = 1.f;
   // What a token needs from memory is asked for one token ahead, so that it travels while the token before is computed.
   struct Fetched { float k, q, x, a, g; };
@@ -287,7 +294,7 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
     f.k = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
     f.q = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
-    f.x = p < a.v_cols ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.v_cols + p) : (p_ok ? 1.f : 0.f);
+    f.x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
     if (a.raw) {
       f.a = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head);
       f.g = 0.f;
@@ -307,22 +314,29 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     if (n + 1 < t_last) next = fetch(MODE == kChunkState ? t - 1 : t + 1);
     const size_t row = (size_t)(q_begin + t);
     const float k_l = cur.k, q_l = cur.q, x = cur.x;
-    float dec, xg;
+    float dec, xg, g;
     if (a.raw) {
       const float z = cur.a + raw_bias;
       const float step = z > 20.f ? z : log1pf(expf(z));
       dec = expf(-rate * step);
-      xg = x * step;
+      g = step;
     } else {
       dec = cur.a;
-      xg = x * cur.g;
+      g = cur.g;
     }
+    xg = x * g;
     if (MODE == kChunkState) {
       const float xw = xg * decays;                       // decays: of the tokens behind t in the chunk
 #pragma unroll
       for (int i = 0; i < NR; ++i) S[i] = fmaf(row_lane(k_l, i), xw, S[i]);
+      if (with_n) nl = fmaf(k_l, g * decays, nl);
       decays *= dec;
       continue;
+    }
+    float nq = 0.f;
+    if (with_n) {
+      nl = fmaf(k_l, g, dec * nl);
+      nq = wave_sum(nl * q_l);
     }
     float y[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -334,27 +348,34 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     float total = (y[0] + y[1]) + (y[2] + y[3]);
     if (waves > 1) {
       part[t & 1][wv][lane] = total;
+      if (with_n && lane == 0) part_n[t & 1][wv] = nq;
       __syncthreads();
       if (wv == 0) {
         total = part[t & 1][0][lane];
         for (int w = 1; w < waves; ++w) total += part[t & 1][w][lane];
+        if (with_n) {
+          nq = part_n[t & 1][0];
+          for (int w = 1; w < waves; ++w) nq += part_n[t & 1][w];
+        }
       }
     }
-    if (wv == 0 && p_ok) a.out[row * (size_t)(a.heads * a.P) + (size_t)head * a.P + p] = fmaf(skip, x, total);
+    if (wv == 0 && p_ok) a.out[row * (size_t)(a.heads * ld) + (size_t)head * ld + p] = fmaf(skip, x, total);
+    if (wv == 0 && with_n && lane == 0) a.out[row * (size_t)(a.heads * ld) + (size_t)head * ld + a.P] = nq;
   }
   if (MODE == kChunkOut) return;
   if (p_ok) {
 #pragma unroll
     for (int i = 0; i < NR; ++i)
-      if (n0 + i < a.N) st[(size_t)(n0 + i) * a.P + p] = S[i];
+      if (n0 + i < a.N) st[(size_t)(n0 + i) * ld + p] = S[i];
   }
+  if (with_n && mine) st[(size_t)(n0 + lane) * ld + a.P] = nl;
   if (MODE == kChunkState && threadIdx.x == 0 && pb == 0) ca.ws_decay[(size_t)blockIdx.y * a.heads + head] = decays;
 }
 
 // Second pass: per sequence and state element, chunk after chunk:  ws[c] <- the state before chunk c,
 // S <- decays[c] * S + S_loc[c];  the state after the last chunk goes to the slot.
 __global__ __launch_bounds__(256) void recurrence_carry_kernel(RecurrenceArgs a, ChunkArgs ca) {
-  const size_t per_head = (size_t)a.N * a.P, per_seq = per_head * a.heads;
+  const size_t per_head = (size_t)a.N * a.ld, per_seq = per_head * a.heads;
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int seq = blockIdx.y;
   if (idx >= per_seq) return;
@@ -385,8 +406,8 @@ static void launch_recurrence(const RecurrenceArgs& a, const ChunkArgs& ca, dim3
   else hipLaunchKernelGGL((linear_recurrence_kernel<64, 256, MODE>), grid, block, 0, stream, a, ca);
 }
 
-// v_cols: P, or P - 1 for a recurrence with a normaliser (v holds P - 1 columns per head; column P - 1 of S and of the output
-// belongs to the constant value 1).
+// v_cols: P, or P - 1 for a recurrence with a normaliser (v holds P - 1 columns per head; column P - 1 of S holds
+// n_t = a_t n_(t-1) + g_t k_t, and the last element of a head's output n_t . q_t).
 // chunk == 0: every sequence token by token in one workgroup per (head, block of channels).  chunk > 0: the three passes
 // over chunks of that many tokens; ws_state holds max_chunks * heads * N * P floats and ws_decay max_chunks * heads, with
 // max_chunks >= sum over the sequences of ceil(q_len / chunk) (total tokens / chunk + num_seqs is enough).
@@ -405,14 +426,14 @@ PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, 
   a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
   a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
   a.raw = raw; a.raw_dtype = raw_dtype; a.raw_stride = raw_stride; a.raw_bias = raw_bias; a.a_log = a_log;
-  a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64; a.v_cols = v_cols;
+  a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = v_cols; a.ld = P; a.pblocks = (v_cols + 63) / 64;
   ChunkArgs ca{ws_state, ws_decay, chunk, num_seqs};
   const int waves = (N + 63) / 64, need = (N + waves - 1) / waves;   // rows of S per wave
   if (chunk == 0) {
     launch_recurrence<kWhole>(a, ca, dim3(heads * a.pblocks, num_seqs), waves, need, stream);
   } else {
     launch_recurrence<kChunkState>(a, ca, dim3(heads * a.pblocks, max_chunks), waves, need, stream);
-    const size_t per_seq = (size_t)heads * N * P;
+    const size_t per_seq = (size_t)heads * N * P;     // (P: all columns of a row of S, the normaliser's among them)
     hipLaunchKernelGGL(recurrence_carry_kernel, dim3((unsigned)((per_seq + 255) / 256), num_seqs), dim3(256), 0, stream, a, ca);
     launch_recurrence<kChunkOut>(a, ca, dim3(heads * a.pblocks, max_chunks), waves, need, stream);
   }
