@@ -468,6 +468,96 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
   }
 }
 
+// Steps of so few pairs that the kernel above would leave most compute units without a workgroup (one request: `top`
+// tiles of one row each): a workgroup is one tile of 16 rows times ONE block of 16 outputs, and its four wavefronts cut
+// K between them in quarters that are multiples of 64; each streams its part of the 16 (gated: 32) weight rows as the
+// kernel above does, two k-steps at a time, and the quarters' sums meet in LDS, where the first wavefront adds them in
+// the quarters' order and stores.  Four times the wavefronts for the same bytes.  An output is the sum of four
+// accumulators instead of one, so it may differ from the other kernels' in the last place; which kernel runs depends
+// on the step's number of pairs alone.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_expert_splitk_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
+                                                                const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
+                                                                int n_out, int K, void* __restrict__ out_, int ld_out, int act,
+                                                                const float* __restrict__ pair_scale) {
+  constexpr int W = GATED ? 2 : 1;
+  __shared__ float part[3][W][4][64];
+  const int tile = blockIdx.x;
+  const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
+  if (nrows <= 0) return;                                    // the whole workgroup: no barrier is left behind
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int block0 = blockIdx.y;
+  const int row = row0 + min(r, nrows - 1);                  // rows past the tile's last repeat it: never stored
+  const bf16* a_ptr = rows_in + (size_t)(GATED ? sorted_pair[row] / top : row) * ld_in + 8 * g;
+  const bf16* we = w + (size_t)expert * W * n_out * K;
+  const int col_r = min(block0 * 16 + r, n_out - 1);         // outputs past the last repeat it: never stored
+  const bf16* w_ptr[W];
+#pragma unroll
+  for (int h = 0; h < W; ++h) w_ptr[h] = we + ((size_t)h * n_out + col_r) * K + 8 * g;
+  const int quarter = ((K + 3) / 4 + 63) & ~63;
+  const int k_begin = min(K, wave * quarter), k_end = min(K, k_begin + quarter);
+  moe_floatx4 acc[W];
+#pragma unroll
+  for (int h = 0; h < W; ++h) acc[h] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int k_pairs = k_begin + ((k_end - k_begin) & ~63);
+#pragma unroll 4
+  for (int k0 = k_begin; k0 < k_pairs; k0 += 64) {
+    moe_bf16x8 a[2], b[W][2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      a[half] = *reinterpret_cast<const moe_bf16x8*>(a_ptr + k0 + 8 * g + 8 * half);
+#pragma unroll
+      for (int h = 0; h < W; ++h) b[h][half] = *reinterpret_cast<const moe_bf16x8*>(w_ptr[h] + k0 + 8 * g + 8 * half);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int h = 0; h < W; ++h) acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[h][half], a[half], acc[h], 0, 0, 0);
+  }
+  // what is left of the last quarter: at most one whole k-step of 32 and a partial one (lanes beyond K hold zeros)
+  for (int k0 = k_pairs; k0 < k_end; k0 += 32) {
+    const bool in = k0 + 8 * g < k_end;
+    const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const moe_bf16x8 a = in ? *reinterpret_cast<const moe_bf16x8*>(a_ptr + k0) : zero;
+#pragma unroll
+    for (int h = 0; h < W; ++h) {
+      const moe_bf16x8 b = in ? *reinterpret_cast<const moe_bf16x8*>(w_ptr[h] + k0) : zero;
+      acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, a, acc[h], 0, 0, 0);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int h = 0; h < W; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave - 1][h][i][lane] = acc[h][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int q = 0; q < 3; ++q)
+#pragma unroll
+    for (int h = 0; h < W; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[h][i] += part[q][h][i][lane];
+  // a lane's four sums: outputs 4 g .. 4 g + 3 of the block, for row r
+  if (r >= nrows) return;
+  const int col = block0 * 16 + 4 * g;
+  if (col >= n_out) return;
+  if (GATED) {
+    bf16* o = reinterpret_cast<bf16*>(out_) + (size_t)(row0 + r) * ld_out + col;
+    const float ps = pair_scale ? pair_scale[sorted_pair[row0 + r]] : 1.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[0][i] * ps, act) * (acc[W - 1][i] * ps));
+  } else {
+    float* o = reinterpret_cast<float*>(out_) + (size_t)(row0 + r) * ld_out + col;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (col + i < n_out) o[i] = acc[0][i];
+  }
+}
+
 // Prompt steps with 128 pairs or more per expert: a workgroup is a tile of 128 rows of one expert times 128 weight rows
 // (gated: 64 of the gate's and the 64 of the up product that belong to them), staged through LDS in k-steps of 64, two
 // buffers deep: every thread fetches eight pieces of 16 bytes of the steps ahead into registers while the matrix cores
@@ -617,8 +707,10 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
   }
 }
 
+constexpr int kSplitBelowWorkgroups = 256;                   // the compute units of the GPU this is written for
+
 template <bool GATED>
-static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, int ld_in, const bf16* w, const int* tiles,
+static void launch_moe_mfma(int tile_rows, int max_tiles, int pairs, const bf16* rows_in, int ld_in, const bf16* w, const int* tiles,
                             const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, const float* pair_scale,
                             hipStream_t stream) {
   const int blocks = (n_out + 15) / 16;
@@ -629,6 +721,10 @@ static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, i
     constexpr int U = GATED ? 1 : 2;
     dim3 grid(max_tiles, (blocks + 4 * U - 1) / (4 * U));
     hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 4, U>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
+  } else if ((long)min(pairs, max_tiles) * ((blocks + 3) / 4) < kSplitBelowWorkgroups && K >= 256) {
+    // at most `pairs` tiles hold a row: too few workgroups of the kernel below to reach every compute unit
+    dim3 grid(max_tiles, blocks);
+    hipLaunchKernelGGL((moe_expert_splitk_kernel<GATED>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
   } else {
     dim3 grid(max_tiles, (blocks + 3) / 4);
     hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 1, 1>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale);
@@ -639,16 +735,17 @@ static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, i
 // as multiplied (it is applied to the gate's and the up product's float sums).
 // tile_rows: what moe_align was given.  Tiles of more than 16 rows are for the matrix-core kernel alone (bfloat16,
 // K and ld_in multiples of 8, 16-byte aligned operands); the plain kernel takes tiles of 16.
+// pairs: how many (token, choice) pairs the tiles hold between them (no more than that many tiles hold a row).
 PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int ld_in, const void* w, const int* tiles, int max_tiles,
-                                  int tile_rows, const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act,
+                                  int tile_rows, const int* sorted_pair, int pairs, int top, int n_out, int K, void* out, int ld_out, int act,
                                   const float* pair_scale, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
-  if (n_out <= 0 || K <= 0 || top <= 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
+  if (n_out <= 0 || K <= 0 || top <= 0 || pairs < 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
   const bool matrix_cores = dtype == PLLM_BF16 && K % 8 == 0 && ld_in % 8 == 0 && ((uintptr_t)rows_in & 15) == 0 && ((uintptr_t)w & 15) == 0;
   if (tile_rows != kMoeTileRows && !(matrix_cores && (tile_rows == 64 || tile_rows == kMoeMaxTileRows))) return -2;
   if (matrix_cores) {
-    if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
-    else launch_moe_mfma<false>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
+    if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, pairs, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
+    else launch_moe_mfma<false>(tile_rows, max_tiles, pairs, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, pair_scale, stream);
     PLLM_RETURN_LAST_ERROR();
   }
   dim3 grid(max_tiles, (n_out + kMoeCols - 1) / kMoeCols), block(256);

@@ -1741,9 +1741,9 @@ def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor,
     _need(pair_scale is None or (gated and pair_scale.dtype == torch.float32 and pair_scale.numel() == pairs and pair_scale.is_contiguous()),
           f"pair_scale: float32 [{pairs}], for the gated product")
     out = torch.empty((pairs, N), dtype=rows_in.dtype if gated else torch.float32, device=rows_in.device)
-    _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
+    _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                                                               c_void_p, c_int, c_int, c_void_p, c_void_p])(
-        dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], tile_rows, _ptr(sorted_pair), top, N, K,
+        dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], tile_rows, _ptr(sorted_pair), pairs, top, N, K,
         _ptr(out), out.stride(0), activation_code(activation), _ptr(pair_scale), _stream()), "moe_expert_gemm")
     return out
 

@@ -52,6 +52,17 @@ class NesezenConfig:
         out.validate()
         return out
 
+    def owner_of(self, i: int) -> int | None:
+        """The layer whose tensors layer i runs with: itself, or where its ``weights_of`` leads (a borrowed layer may be
+        named in turn); None where that leaves the list or never ends."""
+        for _ in range(len(self.layers) + 1):
+            if not 0 <= i < len(self.layers):
+                return None
+            if self.layers[i].weights_of is None:
+                return i
+            i = self.layers[i].weights_of
+        return None
+
     def validate(self) -> None:
         problems = []
         if self.vocab <= 0 or self.width <= 0 or not self.layers:
@@ -62,9 +73,10 @@ class NesezenConfig:
             if l.mlp is not None and l.mlp.get("kind") not in MLP_KINDS:
                 problems.append(f"layer {i}: feed-forward kind {l.mlp.get('kind')!r} is none of {MLP_KINDS}")
             if l.weights_of is not None:
-                if not 0 <= l.weights_of < len(self.layers) or self.layers[l.weights_of].weights_of is not None:
-                    problems.append(f"layer {i}: weights_of names layer {l.weights_of}, which is no layer with weights of its own")
-                elif self.layers[l.weights_of].type != l.type:
+                owner = self.owner_of(i)
+                if owner is None:
+                    problems.append(f"layer {i}: weights_of leads to no layer with weights of its own")
+                elif self.layers[owner].type != l.type:
                     problems.append(f"layer {i}: weights_of names a layer of another type")
         if problems:
             raise ValueError("bad Nesezen config: " + "; ".join(problems))
@@ -121,7 +133,7 @@ def build_spec(cfg: NesezenConfig) -> ModelSpec:
             index_of[i] = len(layers)
             layers.append(LayerSpec(f"l{i}", PartSpec("prenorm_float_stream", names), parts))
     for i, l in enumerate(cfg.layers):
-        schedule.append(ScheduleStep(index_of[i if l.weights_of is None else l.weights_of]))
+        schedule.append(ScheduleStep(index_of[cfg.owner_of(i)]))
     return ModelSpec(
         hidden_size=cfg.width, vocab_size=cfg.vocab,
         embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab, "float_stream": True, "tensor_name": ""}),

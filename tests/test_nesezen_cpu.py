@@ -70,6 +70,18 @@ def test_bad_configurations_are_refused():
             arch.build_spec(arch.read_config(cfg))
 
 
+def test_a_borrowed_layer_may_be_named_in_turn():
+    from paged_llm_amd.config.registry import lookup_architecture
+    arch = lookup_architecture(NESE_A)
+    cfg = copy.deepcopy(NESE_A)
+    cfg["layers"].append(dict(copy.deepcopy(cfg["layers"][3]), weights_of=3))          # 6 -> 3 -> 0
+    spec = arch.build_spec(arch.read_config(cfg))
+    assert [s.layer for s in spec.schedule] == [0, 1, 2, 0, 1, 2, 0] and len(spec.layers) == 3
+    cfg["layers"][3]["weights_of"] = 6                                                 # 3 -> 6 -> 3: never ends
+    with pytest.raises(ValueError):
+        arch.build_spec(arch.read_config(cfg))
+
+
 def test_rotary_frequencies_of_the_engine_are_the_plain_ones():
     """The engine's table builder (frequencies formed in double precision, the rescaling by wavelength) against the
     plain list, for the rescaling's three ranges."""

@@ -187,6 +187,35 @@ def test_experts_with_weights_on_their_inputs_and_a_shared_one(tokens, experts, 
     assert torch.allclose(rows_out.double(), torch.tanh(0.9 * (x0.double() + y)) * w.double() + b.double(), atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("tokens,experts,top", [(1, 8, 2), (2, 5, 1), (3, 4, 4)])
+@pytest.mark.parametrize("W,ff", [(256, 264), (520, 40), (1024, 320)])
+def test_experts_of_steps_with_few_pairs(tokens, experts, top, W, ff):
+    """Steps of one to three tokens, whose products are cut along the inner size between a workgroup's wavefronts: inner
+    sizes of exactly four steps, of no multiple of a step and of several steps a wavefront; outputs that fill no block."""
+    from paged_llm_amd.csrc import ops
+    h = (randn(tokens, W, seed=11) * 0.5).to(torch.bfloat16)
+    wgu = (randn(experts, 2 * ff, W, seed=12) * W ** -0.5).to(torch.bfloat16)
+    wd = (randn(experts, W, ff, seed=13) * ff ** -0.5).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(14)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
+    weights = torch.rand(tokens, top, generator=g) * 0.8 + 0.1
+    rows = ops.moe_tile_rows(ids.numel(), experts, torch.bfloat16, W, ff, W)
+    assert rows == 16
+    sorted_pair, row_of_pair, tiles = ops.moe_align(dev(ids), experts, rows)
+    act = ops.moe_expert_gemm(dev(h), dev(wgu), tiles, sorted_pair, top, True, "silu", tile_rows=rows, pair_scale=dev(weights))
+    out = ops.moe_expert_gemm(act, dev(wd), tiles, sorted_pair, top, False, tile_rows=rows)
+    act, out, where = act.cpu().double(), out.cpu().double(), row_of_pair.cpu().view(tokens, top)
+    for t in range(tokens):
+        for c in range(top):
+            e, row = int(ids[t, c]), int(where[t, c])
+            x = float(weights[t, c]) * h[t].double()
+            a, b = wgu[e, :ff].double() @ x, wgu[e, ff:].double() @ x
+            mid = a / (1.0 + torch.exp(-a)) * b
+            assert float((act[row] - mid).abs().max()) <= 1e-2 * float(mid.abs().max()) + 1e-6, ("gated", t, c)
+            want = wd[e].double() @ act[row]
+            assert float((out[row] - want).abs().max()) <= 1e-5 * float(want.abs().max()) + 1e-7, ("down", t, c)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_latent_preparation_from_float_sums_with_a_latent_of_the_queries(dtype):
     from paged_llm_amd.csrc import ops
