@@ -252,3 +252,24 @@ def test_the_whole_model_is_the_sum_of_its_branches():
             x = x + (plain.gated_feed_forward(h, wf) if l["mlp"]["kind"] == "dense" else plain.routed_feed_forward(h, wf, l["mlp"]))
         assert torch.allclose(seen[i], x, atol=1e-6)
     assert not torch.allclose(seen[0], seen[3]) and not torch.allclose(seen[1], seen[4])
+
+
+def test_the_configuration_that_bench_measures_builds():
+    """``bench.py --nesezen`` measures a configuration of its own making: it passes the registry and has the layers
+    its description names."""
+    import os
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if root not in sys.path:
+        sys.path.insert(0, root)
+    import bench
+    from paged_llm_amd.config.registry import lookup_architecture
+    for width in (1024, 2048):
+        cfg = bench.nesezen_config(width, 32000)
+        arch = lookup_architecture(cfg)
+        spec = arch.build_spec(arch.read_config(cfg))
+        assert len(spec.schedule) == len(spec.layers) == 12 and spec.hidden_size == width
+        kinds = [l.parts["mixer"].kind for l in spec.layers]
+        assert kinds.count("normed_attention") == 6 and kinds.count("mlstm") == 3 and kinds.count("latent_attention") == 3
+        assert sum(l.parts["feed_forward"].kind == "routed_experts" for l in spec.layers) == 6
+
