@@ -105,7 +105,7 @@ def _mixer_spec(kind: str, m: dict, eps: float) -> PartSpec:
         return PartSpec("mlstm", {"heads": int(m["heads"]), "key_dim": int(m["dim"]), "head_dim": int(m["vdim"]),
                                   "gate_cap": float(m.get("gate_cap") or 0.0), "eps": eps})
     return PartSpec("latent_attention", {"heads": int(m["heads"]), "plain_dim": int(m["dim"]), "rot_dim": 0, "head_dim": int(m["vdim"]),
-                                         "rank": int(m["kv_rank"]), "q_rank": int(m.get("q_rank") or 0), "scale": float(m["scale"]), "window": 0,
+                                         "rank": int(m["kv_rank"]), "q_rank": int(m["q_rank"]), "scale": float(m["scale"]), "window": 0,
                                          "position": None, "eps": eps, "head_gate": True})
 
 
