@@ -42,12 +42,15 @@ class GroupSpec:
     name: str
     kind: str = "full"        # "full" | "window" | "chunk"
     window: int = 0           # positions kept, for kind "window"; positions of a block, for kind "chunk"
+    keep_first: int = 0       # kind "window": the sequence's first positions that every later query still sees; their pages stay
 
     def __post_init__(self):
         if self.kind not in ("full", "window", "chunk"):
             raise ValueError(f"unknown cache group kind {self.kind!r}")
         if self.kind != "full" and self.window <= 0:
             raise ValueError("a windowed or chunked group needs window > 0")
+        if self.keep_first < 0 or (self.keep_first > 0 and self.kind != "window"):
+            raise ValueError("first positions are kept beside a sliding window only, and their number is not negative")
 
 
 @dataclass(frozen=True)
@@ -307,6 +310,10 @@ class CacheManager:
         """Pages below this index are out of the window of every query at position >= num_computed."""
         return first_visible_key(g.kind, g.window, num_computed) // self.block_size
 
+    def _kept_pages(self, g: GroupSpec) -> int:
+        """Pages at the start of a table that a window never passes: those that hold the kept first positions."""
+        return (g.keep_first + self.block_size - 1) // self.block_size
+
     def _nothing_to_do(self, hold: _Holding, num_computed: int, num_new: int, total_pages: int) -> bool:
         """The usual decode step: the pages are there, the one written to is the request's alone, and
         no window has moved past a page."""
@@ -351,14 +358,14 @@ class CacheManager:
                     if page != NO_PAGE and pool.refs[page] + (1 if idx >= len(table) else 0) > 1:
                         cow_index = idx
             # Pages a window has passed come back before the new ones are taken.
-            first_needed = self._first_needed_page(g, num_computed)
-            releasable = [i for i in range(min(first_needed, len(table))) if table[i] != NO_PAGE
+            first_needed, kept = self._first_needed_page(g, num_computed), self._kept_pages(g)
+            releasable = [i for i in range(kept, min(first_needed, len(table))) if table[i] != NO_PAGE
                           and pool.refs[table[i]] == 1]
             revive = sum(1 for p in hits if pool.refs[p] == 0)
             available = pool.num_free - revive + len(releasable)
             if need + (1 if cow_index is not None else 0) > available:
                 return False
-            plan[name] = (hits, need, cow_index, first_needed)
+            plan[name] = (hits, need, cow_index, first_needed, kept)
         if new_request and self.uses_state and self.slots.num_free == 0:
             return False
 
@@ -368,10 +375,10 @@ class CacheManager:
                 hold.state_slot = self.slots.acquire()
             self._held[request] = hold
         changed = new_request
-        for name, (hits, need, cow_index, first_needed) in plan.items():
+        for name, (hits, need, cow_index, first_needed, kept) in plan.items():
             pool, table = self.pools[name], hold.tables[name]
             changed = changed or bool(hits) or need > 0 or cow_index is not None
-            for i in range(min(first_needed, len(table))):
+            for i in range(kept, min(first_needed, len(table))):
                 if table[i] != NO_PAGE:
                     pool.drop(table[i])
                     table[i] = NO_PAGE
@@ -381,7 +388,7 @@ class CacheManager:
             table.extend(hits)
             for i in range(need):
                 # A page that lies wholly before the window is never written or read.
-                table.append(pool.take() if len(table) >= first_needed else NO_PAGE)
+                table.append(pool.take() if len(table) >= first_needed or len(table) < kept else NO_PAGE)
             if cow_index is not None:
                 shared = table[cow_index]
                 fresh = pool.take()

@@ -10,6 +10,9 @@
 // Query i of a sequence sits at position seq_len_k - num_q + i and sees keys n <= that position
 // (and n > position - window when window > 0; with window < 0, only the keys of its own block of -window positions).  Query head j reads kv head j / (heads / kv_heads).
 // A score may carry further terms (a cap, a slope times the distance, a sink per head: ScoreTerms).
+// keep_first > 0: the sequence's first keep_first positions stay visible to every later query, whatever the window
+// (they keep their own positions: nothing about their keys changes).
+// weighting 1: no softmax; a visible key weighs sigmoid(score + head_bias[head]) and the weights are not normalised.
 //
 // Keys are walked in tiles of 64 aligned to absolute positions 0, 64, 128, ..., so the order of
 // every sum for one (token, head) is the same however the tokens were cut into steps or batched.
@@ -25,7 +28,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     T* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_seqs, int num_heads,
-    int num_kv_heads, int head_dim, int block_size, float scale, int window, ScoreTerms terms) {
+    int num_kv_heads, int head_dim, int block_size, float scale, int window, ScoreTerms terms, int keep_first, int weighting,
+    const float* __restrict__ head_bias) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float p_s[64];
   __shared__ int page_s[64];
@@ -55,9 +59,14 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
   if (terms.sinks) { m = terms.sinks[head]; l = 1.f; }          // as if one key with this score and no value had been seen
   const float slope = terms.slopes ? terms.slopes[head] : 0.f;
 
-  for (int n0 = (first_key / 64) * 64; n0 <= q_pos; n0 += 64) {
+  const float bias_h = (weighting == 1 && head_bias) ? head_bias[head] : 0.f;
+  for (int n0 = keep_first > 0 ? 0 : (first_key / 64) * 64; n0 <= q_pos; n0 += 64) {
+    if (n0 >= keep_first && n0 + 63 < first_key) {            // a tile between the kept positions and the window: on to the window's first
+      n0 = (first_key / 64) * 64 - 64;
+      continue;
+    }
     const int n = n0 + lane;
-    const bool visible = n >= first_key && n <= q_pos;
+    const bool visible = n <= q_pos && (n >= first_key || n < keep_first);
     float s = -INFINITY;
     int page = 0;
     if (visible) {
@@ -68,11 +77,16 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       s = capped_score(dot * scale, terms.cap);
       if (terms.slopes) s += slope * (float)(n - q_pos);
     }
-    const float m_new = fmaxf(m, wave_max(s));   // finite: the tile holds at least one visible key
-    const float alpha = expf(m - m_new);          // 0 on the first tile (without a sink)
-    const float p = visible ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(p);
-    m = m_new;
+    float alpha = 1.f, p;
+    if (weighting == 1) {
+      p = visible ? 1.f / (1.f + expf(-(s + bias_h))) : 0.f;
+    } else {
+      const float m_new = fmaxf(m, wave_max(s));   // finite: the tile holds at least one visible key
+      alpha = expf(m - m_new);                      // 0 on the first tile (without a sink)
+      p = visible ? expf(s - m_new) : 0.f;
+      l = l * alpha + wave_sum(p);
+      m = m_new;
+    }
     __syncthreads();
     p_s[lane] = p;
     page_s[lane] = page;
@@ -94,7 +108,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       acc[r] = a;
     }
   }
-  const float inv_l = 1.f / l;
+  const float inv_l = weighting == 1 ? 1.f : 1.f / l;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int i = lane + r * 64;
@@ -108,19 +122,21 @@ PLLM_API int pllm_paged_attention_generic(int dtype, const void* q, int q_stride
                                           const int* cu_seqlens_q, const int* seq_lens_k, int num_seqs, int total_q,
                                           int num_heads, int num_kv_heads, int head_dim, int block_size, float scale,
                                           int window, float score_cap, const float* slopes, const float* sinks,
-                                          hipStream_t stream) {
+                                          int keep_first, int weighting, const float* head_bias, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (head_dim > kMaxHeadDim || head_dim <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
-  if (!(score_cap >= 0.f)) return -2;
+  if (!(score_cap >= 0.f) || keep_first < 0 || weighting < 0 || weighting > 1 || (keep_first > 0 && window < 0)) return -2;
   const ScoreTerms terms{score_cap, slopes, sinks};
   dim3 grid(total_q, num_heads), block(64);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_stride,
                        (const float*)k_pages, (const float*)v_pages, (float*)out, out_stride, block_tables, bt_stride,
-                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms);
+                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms, keep_first,
+                       weighting, head_bias);
   else
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16>, grid, block, 0, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride,
-                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms);
+                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms, keep_first,
+                       weighting, head_bias);
   PLLM_RETURN_LAST_ERROR();
 }

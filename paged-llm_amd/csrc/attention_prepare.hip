@@ -5,7 +5,9 @@
 //                     over time on every channel (inputs of earlier steps from the request's state slot), rotary
 //                     encoding of the first rot elements of q and k heads (pairs (i, i + rot/2) or (2i, 2i + 1)),
 //                     q and k divided by their root mean square over the head (unless qk_norm is 0), q written as rows of padded heads,
-//                     k and v written into their cache pages;
+//                     k and v written into their cache pages; the values as projected (v_mode 0), divided by their root
+//                     mean square over the head (1), or the keys as they were before their rotation, the product
+//                     holding no value columns at all (2);
 //   conv_inputs_keep  leaves the last taps - 1 projected rows of every sequence in its state slot;
 //   gate_heads        out[t, h, :dv] = o[t, h, :dv] * sigmoid(gate[t, h]) from padded heads to packed ones.
 //
@@ -29,7 +31,7 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
     const float* __restrict__ proj, int ld, const float* __restrict__ bias, const float* __restrict__ conv_w, int taps,
     const float* __restrict__ state, size_t slot_stride, const int* __restrict__ state_slots, const int* __restrict__ seq_starts,
     const int* __restrict__ cu_seqlens, int num_seqs, const int* __restrict__ positions, const float* __restrict__ cos_table,
-    const float* __restrict__ sin_table, int rot, int interleaved, float eps, int qk_norm, int heads, int kv_heads, int d, int dv, int D,
+    const float* __restrict__ sin_table, int rot, int interleaved, float eps, int qk_norm, int v_mode, int heads, int kv_heads, int d, int dv, int D,
     T* __restrict__ q_out, const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int block_size) {
   __shared__ float vals[kPrepMaxHead];
   const int lane = threadIdx.x;
@@ -38,8 +40,9 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
   int kind, head, base, width;
   if (hs < heads) { kind = 0; head = hs; base = hs * d; width = d; }
   else if (hs < heads + kv_heads) { kind = 1; head = hs - heads; base = heads * d + head * d; width = d; }
+  else if (v_mode == 2) { kind = 2; head = hs - heads - kv_heads; base = heads * d + head * d; width = d; }
   else { kind = 2; head = hs - heads - kv_heads; base = (heads + kv_heads) * d + head * dv; width = dv; }
-  const int channels = (heads + kv_heads) * d + kv_heads * dv;
+  const int channels = (heads + kv_heads) * d + (v_mode == 2 ? 0 : kv_heads * dv);
 
   int q_begin = 0, carried = 0;
   const float* st = nullptr;
@@ -106,6 +109,15 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
       for (int r = 0; r < 4; ++r) x[r] *= inv;
     }
   }
+  if (kind == 2 && v_mode == 1) {
+    float sq = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (lane + 64 * r < width) sq = fmaf(x[r], x[r], sq);
+    const float inv = 1.f / sqrtf(wave_sum(sq) / (float)width + eps);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) x[r] *= inv;
+  }
   if (kind == 0) {
     T* out = q_out + ((size_t)tok * heads + head) * D;
 #pragma unroll
@@ -165,22 +177,23 @@ __global__ __launch_bounds__(256) void conv_inputs_keep_kernel(
 PLLM_API int pllm_attn_prepare(int dtype, const float* proj, int ld, const float* bias, const float* conv_w, int taps, float* state,
                                long slot_stride, const int* state_slots, const int* seq_starts, const int* cu_seqlens, int num_seqs,
                                const int* positions, const float* cos_table, const float* sin_table, int rot, int interleaved,
-                               float eps, int qk_norm, int heads, int kv_heads, int d, int dv, int D, void* q_out, const int* slot_mapping,
+                               float eps, int qk_norm, int v_mode, int heads, int kv_heads, int d, int dv, int D, void* q_out, const int* slot_mapping,
                                void* k_pages, void* v_pages, int block_size, int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || dv <= 0 || d > D || dv > D || D > kPrepMaxHead || rot < 0 || rot > d || (rot & 1) || taps > kPrepMaxTaps) return -2;
+  if (v_mode < 0 || v_mode > 2 || (v_mode == 2 && dv != d)) return -2;
   if (rot > 0 && (!cos_table || !sin_table)) return -2;
   if (taps > 1 && (!conv_w || !state || !state_slots || !seq_starts || !cu_seqlens)) return -2;
   const bool write = slot_mapping && k_pages && v_pages;
   dim3 grid(num_tokens, heads + (write ? 2 * kv_heads : 0)), block(64);
 #define PLLM_PREP(T)                                                                                                              \
   hipLaunchKernelGGL(attn_prepare_kernel<T>, grid, block, 0, stream, proj, ld, bias, conv_w, taps, state, (size_t)slot_stride,   \
-                     state_slots, seq_starts, cu_seqlens, num_seqs, positions, cos_table, sin_table, rot, interleaved, eps, qk_norm, heads, \
+                     state_slots, seq_starts, cu_seqlens, num_seqs, positions, cos_table, sin_table, rot, interleaved, eps, qk_norm, v_mode, heads, \
                      kv_heads, d, dv, D, (T*)q_out, slot_mapping, (T*)k_pages, (T*)v_pages, block_size)
   if (dtype == PLLM_F32) PLLM_PREP(float); else PLLM_PREP(bf16);
 #undef PLLM_PREP
   if (taps > 1) {
-    const int channels = (heads + kv_heads) * d + kv_heads * dv;
+    const int channels = (heads + kv_heads) * d + (v_mode == 2 ? 0 : kv_heads * dv);
     dim3 g2((channels + 255) / 256, num_seqs);
     hipLaunchKernelGGL(conv_inputs_keep_kernel, g2, dim3(256), 0, stream, proj, ld, bias, state, (size_t)slot_stride, state_slots,
                        seq_starts, cu_seqlens, channels, taps);

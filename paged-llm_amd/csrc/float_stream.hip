@@ -34,6 +34,65 @@ PLLM_API int pllm_embed_scaled(int dtype, const int* ids, const void* table, flo
 }
 
 // ---------------------------------------------------------------------------------------------
+// A token embedding with a hashed bigram row added:
+//   x[t, :] = float(table[ids[t], :]) * scale + float(pairs[row(t), :]),
+//   row(t) = (previous token * mul_prev + ids[t] * mul_cur) mod buckets, or `buckets` (the table's last row) for a
+//   sequence's first token.
+// The token before a step's first token of a sequence is what the sequence's slot of `last_token` holds (a sequence
+// whose seq_starts is 0 has none); every sequence leaves its last token of this step there.  bigram_rows_kernel: one
+// workgroup per sequence, which reads the slot before any of its threads writes it.
+__global__ __launch_bounds__(256) void bigram_rows_kernel(const int* __restrict__ ids, const int* __restrict__ cu_seqlens,
+                                                          const int* __restrict__ seq_starts, const int* __restrict__ state_slots,
+                                                          int* last_token, long slot_stride, int* __restrict__ rows, int vocab,
+                                                          int buckets, int mul_prev, int mul_cur) {
+  const int seq = blockIdx.x;
+  const int begin = cu_seqlens[seq], len = cu_seqlens[seq + 1] - begin;
+  if (len <= 0) return;
+  int* slot = last_token + (size_t)state_slots[seq] * slot_stride;
+  const int carried = seq_starts[seq] > 0 ? *slot : -1;
+  __syncthreads();
+  for (int i = threadIdx.x; i < len; i += blockDim.x) {
+    const int cur = ids[begin + i];
+    const int prev = i > 0 ? ids[begin + i - 1] : carried;
+    int row = buckets;
+    if (prev >= 0) row = (int)(((long long)prev * mul_prev + (long long)cur * mul_cur) % buckets);
+    rows[begin + i] = row < 0 ? row + buckets : row;
+    if (i == len - 1) *slot = cur;
+  }
+}
+
+template <typename T>
+__global__ void embed_bigram_kernel(const int* __restrict__ ids, const int* __restrict__ pair_rows, const T* __restrict__ table,
+                                    const T* __restrict__ pairs, float* __restrict__ x, int hidden, int vocab, int buckets, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t], pr = pair_rows[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never fault
+  pr = pr < 0 ? 0 : (pr > buckets ? buckets : pr);
+  const T* src = table + (size_t)id * hidden;
+  const T* add = pairs + (size_t)pr * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) x[(size_t)t * hidden + i] = to_f32(src[i]) * scale + to_f32(add[i]);
+}
+
+PLLM_API int pllm_embed_bigram(int dtype, const int* ids, const int* cu_seqlens, const int* seq_starts, const int* state_slots,
+                               int* last_token, long slot_stride, int* pair_rows, const void* table, const void* pairs, float* x,
+                               int num_tokens, int num_seqs, int hidden, int vocab, int buckets, int mul_prev, int mul_cur, float scale,
+                               int move_state, hipStream_t stream) {
+  if (num_tokens <= 0 || num_seqs <= 0) return 0;
+  if (buckets <= 0 || hidden <= 0) return -2;
+  if (move_state)
+    hipLaunchKernelGGL(bigram_rows_kernel, dim3(num_seqs), dim3(256), 0, stream, ids, cu_seqlens, seq_starts, state_slots, last_token,
+                       slot_stride, pair_rows, vocab, buckets, mul_prev, mul_cur);
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(embed_bigram_kernel<float>, grid, block, 0, stream, ids, pair_rows, (const float*)table, (const float*)pairs, x,
+                       hidden, vocab, buckets, scale);
+  else
+    hipLaunchKernelGGL(embed_bigram_kernel<bf16>, grid, block, 0, stream, ids, pair_rows, (const bf16*)table, (const bf16*)pairs, x,
+                       hidden, vocab, buckets, scale);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
 // Layer norm of one row per workgroup:  y = (v - mean) / sqrt(var + eps) * w + b,  var = mean((v - mean)^2),
 // with v = in[src] (src = row_index[r] or r).  Then
 //   stream given:  stream[r] += y (float), and rows[r] = T(stream[r]) when rows is given;
@@ -183,6 +242,7 @@ PLLM_API int pllm_round_rows(const float* x, void* rows, long n, hipStream_t str
 // ---------------------------------------------------------------------------------------------
 // RMS norms on both sides of a branch over a float stream, one row per workgroup:
 //   branch given:  y = branch[r] (+ bias);  stream[r] += mult * y / sqrt(mean(y^2) + eps) * w_branch      (in place)
+//                  (w_branch null: the branch is not normed, stream[r] += mult * y: a pre-norm block's sum)
 //   then, rows given:  rows[r] = T(s / sqrt(mean(s^2) + eps) * w_next)  with s the row of the stream as it is now
 //                      (w_next null: rows[r] = T(s), the stream in the compute type).
 // Without a branch the stream's row is src = row_index[r] (or r) and nothing is written to the stream.  The weights
@@ -208,9 +268,9 @@ __global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restri
       row[i] = f;
       bsq = fmaf(f, f, bsq);
     }
-    const float inv = 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps);
+    const float inv = w_branch ? 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps) : 1.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float y = s[i] + mult * (row[i] * inv * w_branch[i]);
+      const float y = s[i] + mult * (w_branch ? row[i] * inv * w_branch[i] : row[i]);
       s[i] = y;
       row[i] = y;
       sq = fmaf(y, y, sq);
@@ -257,7 +317,7 @@ __global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const f
     const int i = tid + kHeldThreads * j;
     const bool in = i < hidden;
     sv[j] = in ? s[i] : 0.f;
-    wb[j] = in ? w_branch[i] : 0.f;
+    wb[j] = (in && w_branch) ? w_branch[i] : 1.f;
     wn[j] = (in && w_next) ? w_next[i] : 1.f;
     f[j] = (in && !sum.expert_out) ? branch[(size_t)r * hidden + i] : 0.f;
   }
@@ -283,13 +343,13 @@ __global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const f
       bsq = fmaf(f[j], f[j], bsq);
     }
   }
-  const float inv = 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps);
+  const float inv = w_branch ? 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps) : 1.f;
   float sq = 0.f;
 #pragma unroll
   for (int j = 0; j < kHeldPerThread; ++j) {
     const int i = tid + kHeldThreads * j;
     if (i < hidden) {
-      const float y = sv[j] + mult * (f[j] * inv * wb[j]);
+      const float y = sv[j] + mult * (w_branch ? f[j] * inv * wb[j] : f[j]);
       s[i] = y;
       sv[j] = y;
       sq = fmaf(y, y, sq);
@@ -333,7 +393,7 @@ PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* 
                                const int* row_index, const float* w_next, float eps, void* rows, long rows_stride, int num_rows,
                                int hidden, hipStream_t stream_) {
   if (num_rows <= 0) return 0;
-  if (hidden <= 0 || !stream || (branch && !w_branch)) return -2;
+  if (hidden <= 0 || !stream) return -2;
   if (branch && hidden <= kHeldPerThread * kHeldThreads) {
     const ChoiceSum none{nullptr, nullptr, 0, nullptr, nullptr, 0};
     if (out_dtype == PLLM_F32) launch_sandwich_held<float>(PLLM_F32, branch, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
@@ -555,5 +615,24 @@ PLLM_API int pllm_dyt_sum(int out_dtype, int h_dtype, const float* expert_out, c
   if (out_dtype == PLLM_F32) { if (h_dtype == PLLM_F32) PLLM_DS(float, float); else PLLM_DS(float, bf16); }
   else { if (h_dtype == PLLM_F32) PLLM_DS(bf16, float); else PLLM_DS(bf16, bf16); }
 #undef PLLM_DS
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out = sa * a + sb * b, element by element in float: two mixers' outputs that enter the stream as one branch.
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_sum_kernel(const T* __restrict__ a, float sa, const T* __restrict__ b, float sb,
+                                                         T* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(sa * to_f32(a[i]) + sb * to_f32(b[i]));
+}
+
+PLLM_API int pllm_scaled_sum(int dtype, const void* a, float sa, const void* b, float sb, void* out, long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(scaled_sum_kernel<float>, grid, block, 0, stream, (const float*)a, sa, (const float*)b, sb, (float*)out, (size_t)n);
+  else
+    hipLaunchKernelGGL(scaled_sum_kernel<bf16>, grid, block, 0, stream, (const bf16*)a, sa, (const bf16*)b, sb, (bf16*)out, (size_t)n);
   PLLM_RETURN_LAST_ERROR();
 }

@@ -78,7 +78,7 @@ _SIGNATURES = {
     "pllm_gemm_nt": [c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_paged_attention_generic": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                     c_float, c_void_p, c_void_p, c_void_p],
+                                     c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "pllm_sample": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_ulonglong, c_void_p,
                     c_void_p, c_void_p],
     "pllm_sample_workspace_bytes": [c_int, c_int],
@@ -303,6 +303,35 @@ class ScoreTerms:
         return self
 
 
+class KeyWeights:
+    """How the visible keys of a query are chosen and weighed where that differs from a causal window under a softmax
+    (None everywhere else):
+
+    * ``keep_first`` k > 0: the sequence's first k positions stay visible to every later query whatever the window
+      (query i sees key j when j <= i and (i - j < window or j < k)); the kept keys are at their own positions;
+    * ``sigmoid``: no softmax; a visible key weighs sigmoid(score + ``head_bias[h]``) (float32 [heads] on the device, or
+      None for no bias) and the weights are not normalised over the keys."""
+
+    __slots__ = ("keep_first", "sigmoid", "head_bias")
+
+    def __init__(self, keep_first: int = 0, sigmoid: bool = False, head_bias: torch.Tensor | None = None):
+        self.keep_first, self.sigmoid, self.head_bias = int(keep_first), bool(sigmoid), head_bias
+
+    def any(self) -> bool:
+        return self.keep_first > 0 or self.sigmoid
+
+    def checked(self, num_heads: int, window: int, device) -> "KeyWeights":
+        _need(self.keep_first >= 0, f"kept first positions: a count >= 0, got {self.keep_first}")
+        _need(self.keep_first == 0 or window >= 0, "first positions are kept beside a sliding window, not beside blocks")
+        _need(self.head_bias is None or self.sigmoid, "a bias per head belongs to sigmoid weights")
+        if self.head_bias is not None:
+            t = self.head_bias
+            _on_gpu(t)
+            _need(t.dtype == torch.float32 and t.shape == (num_heads,) and t.is_contiguous() and t.device == device,
+                  f"head_bias: float32 [{num_heads}] beside the queries")
+        return self
+
+
 def _terms_args(terms: "ScoreTerms | None", num_heads: int, device) -> tuple:
     if terms is None:
         return c_float(0.0), None, None
@@ -313,7 +342,7 @@ def _terms_args(terms: "ScoreTerms | None", num_heads: int, device) -> tuple:
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                             cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                             head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
-                            terms: ScoreTerms | None = None) -> torch.Tensor:
+                            terms: ScoreTerms | None = None, weights: KeyWeights | None = None) -> torch.Tensor:
     """Causal attention over paged keys and values; one wavefront per (token, head), all in float.
 
     The caller guarantees (and the step function checks on the host) that every table entry
@@ -322,6 +351,8 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
     _need(0 < head_dim <= MAX_HEAD_DIM_GENERIC, f"attention kernel takes head sizes up to {MAX_HEAD_DIM_GENERIC}, got {head_dim}")
     _need(num_heads <= 65535, "too many heads for one launch")
+    if weights is not None:
+        weights.checked(num_heads, int(window or 0), q.device)
     T = q.shape[0]
     if out is None:
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
@@ -329,7 +360,8 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _check(_fn("attention_generic.hip", "pllm_paged_attention_generic")(
         dtype_code(q.dtype), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0),
         _ptr(block_tables), block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, num_heads, num_kv_heads,
-        head_dim, bs, c_float(scale), int(window or 0), *_terms_args(terms, num_heads, q.device), _stream()),
+        head_dim, bs, c_float(scale), int(window or 0), *_terms_args(terms, num_heads, q.device),
+        *((weights.keep_first, int(weights.sigmoid), _ptr(weights.head_bias)) if weights is not None else (0, 0, None)), _stream()),
         "paged_attention_generic")
     return out
 
@@ -992,7 +1024,7 @@ SPLIT_FROM_CONTEXT_TIMES_HEAD = 160_000   # context x head size of a few-query s
 
 
 def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
-                    scale, window, ctx, terms: ScoreTerms | None = None) -> torch.Tensor:
+                    scale, window, ctx, terms: ScoreTerms | None = None, weights: KeyWeights | None = None) -> torch.Tensor:
     """Attention of one step's queries over the paged cache: the MFMA kernels for bfloat16 where they
     take the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions.
 
@@ -1003,6 +1035,9 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     their keys into partitions, the portions to the prompt kernel (a portion of 512 tokens beside 7 decoded tokens
     at context 8192: 109 us in one launch, 36 us in two; at context 1024: 19 us and 24 us)."""
     bs = k_pages.shape[2]
+    if weights is not None and weights.any():
+        return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
+                                       scale, window, terms=terms, weights=weights)
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
         group = num_heads // num_kv_heads
         lds = _max_lds_bytes(q.device)
@@ -1081,6 +1116,34 @@ def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, want_rows
     _check(_fn("float_stream.hip", "pllm_embed_scaled", signature=sig)(dtype_code(table.dtype), _ptr(ids), _ptr(table), _ptr(x), _ptr(rows),
                                                                       T, H, V, c_float(scale), _stream()), "embed_scaled")
     return x, rows
+
+
+def embed_bigram(ids: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor, scale: float, buckets: int, mul_prev: int, mul_cur: int,
+                 state: torch.Tensor, state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
+                 pair_rows: torch.Tensor, move_state: bool = True) -> torch.Tensor:
+    """float32 [T, hidden]: x[t] = float(table[ids[t]]) * scale + float(pairs[row(t)]) with row(t) = (token before * mul_prev +
+    ids[t] * mul_cur) mod buckets, or ``buckets`` for a sequence's first token.  The token before a step's first token of a
+    sequence is ``state[slot, 0]`` (int32 [slots, 1]; none when seq_starts == 0), where every sequence leaves its last token
+    of this step.  ``pair_rows`` int32 [T] receives the rows; with ``move_state`` False it is read instead (a second
+    gather of the same step) and the state stays as it is."""
+    _on_gpu(ids, table, pairs, state, state_slots, seq_starts, cu_seqlens, pair_rows)
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be contiguous int32 [T]")
+    T, (V, H) = ids.numel(), table.shape
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    _need(pairs.shape == (buckets + 1, H) and pairs.is_contiguous() and pairs.dtype == table.dtype, f"bigram table: [{buckets + 1}, {H}] of the token table's type")
+    _need(state.dtype == torch.int32 and state.dim() == 2 and state.is_contiguous(), "the last tokens' state is contiguous int32 [slots, 1]")
+    for t, n, what in ((state_slots, num_seqs, "state_slots"), (seq_starts, num_seqs, "seq_starts"), (cu_seqlens, num_seqs + 1, "cu_seqlens")):
+        _need(t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous() and t.numel() == n, f"{what} must be contiguous int32 [{n}]")
+    _need(pair_rows.dtype == torch.int32 and pair_rows.numel() == T and pair_rows.is_contiguous(), "pair_rows: int32 [T]")
+    _need(0 < buckets and abs(mul_prev) < 2 ** 31 and abs(mul_cur) < 2 ** 31, "bigram hash: buckets > 0 and 32-bit multipliers")
+    x = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    sig = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+           c_int, c_int, c_int, c_float, c_int, c_void_p]
+    _check(_fn("float_stream.hip", "pllm_embed_bigram", signature=sig)(
+        dtype_code(table.dtype), _ptr(ids), _ptr(cu_seqlens), _ptr(seq_starts), _ptr(state_slots), _ptr(state), state.stride(0), _ptr(pair_rows),
+        _ptr(table), _ptr(pairs), _ptr(x), T, num_seqs, H, V, buckets, mul_prev, mul_cur, c_float(scale), int(bool(move_state)), _stream()),
+        "embed_bigram")
+    return x
 
 
 def layernorm(v: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, stream_rows: torch.Tensor | None = None,
@@ -1245,7 +1308,7 @@ def recurrence_chunk(max_q_len: int, num_tokens: int) -> int:
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, state_offset: int,
                       state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
                       vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None, max_q_len: int = 0,
-                      step_sizes: tuple | None = None, normaliser: bool = False) -> torch.Tensor:
+                      step_sizes: tuple | None = None, normaliser: bool = False, row_decay: torch.Tensor | None = None) -> torch.Tensor:
     """Per head:  S_t = decay_t S_(t-1) + k_t (vscale_t v_t)^T,   y_t = S_t^T q_t + skip v_t,   S [N, P] float32 at
     ``state[slot, state_offset + head * N * P :]``; a sequence with seq_starts == 0 starts from S = 0.
 
@@ -1256,6 +1319,8 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     ``decay`` (None) and ``vscale``: the kernel makes vscale_t = softplus(raw_t + bias) and decay_t = exp(-exp(a_log) vscale_t) itself.
     ``normaliser``: S has one more column, P + 1, whose value is 1 at every token (it holds n_t = decay_t n_(t-1) + vscale_t k_t);
     the state then takes heads * N * (P + 1) floats and y is [T, heads * (P + 1)] with n_t . q_t in every head's last column.
+    ``row_decay`` float32 [T, heads, N] (a view, heads side by side, unit inner stride) in place of ``decay`` (None): a decay per
+    row of S, S_t = diag(row_decay_t) S_(t-1) + k_t (vscale_t v_t)^T (every head then has its own keys).
     ``max_q_len``: a bound on the tokens of one sequence in this step (0: unknown); from ``RECURRENCE_CHUNKS_FROM`` on the
     sequences are cut into chunks that run side by side (a chunk's own contribution from a zero state, the states carried
     from chunk to chunk, the outputs from each chunk's true starting state), which rounds differently than token by token."""
@@ -1275,6 +1340,11 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
         _need(raw.shape == (T, H) and raw.stride(1) == 1, f"raw step sizes: [{T}, {H}] with unit inner stride")
         for t in (raw_bias, a_log):
             _need(t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"step sizes: float32 [{H}] per-head constants")
+    elif row_decay is not None:
+        _on_gpu(row_decay)
+        _need(decay is None and KH == H, "a decay per row takes the place of the decay per head, and every head has its own keys")
+        _need(row_decay.dtype == torch.float32 and tuple(row_decay.shape) == (T, H, N) and row_decay.stride(2) == 1 and row_decay.stride(1) == N,
+              f"row_decay: float32 [{T}, {H}, {N}] with the heads side by side")
     else:
         _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) in ((T, H), (H,)), f"decay: float32 [{T}, {H}] or [{H}]")
     _need(vscale is None or (vscale.dtype == torch.float32 and vscale.shape == (T, H) and vscale.is_contiguous()), f"vscale: float32 [{T}, {H}]")
@@ -1285,35 +1355,76 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     chunk = recurrence_chunk(max_q_len, T)
     max_chunks = T // chunk + num_seqs if chunk else 0
     ws_state = torch.empty((max_chunks, H * N * P), dtype=torch.float32, device=v.device) if chunk else None
-    ws_decay = torch.empty((max_chunks, H), dtype=torch.float32, device=v.device) if chunk else None
-    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+    ws_decay = torch.empty((max_chunks, H * (N if row_decay is not None else 1)), dtype=torch.float32, device=v.device) if chunk else None
+    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
            c_void_p, c_int, c_int, c_void_p, c_void_p,
            c_void_p, c_long, c_void_p, c_void_p,
            c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     _check(_fn("recurrent.hip", "pllm_linear_recurrence", signature=sig)(
         _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay),
-        H if decay is not None and decay.dim() == 2 else 0, _ptr(vscale), _ptr(skip),
+        H if decay is not None and decay.dim() == 2 else 0, _ptr(row_decay), row_decay.stride(0) if row_decay is not None else 0,
+        _ptr(vscale), _ptr(skip),
         _ptr(raw), dtype_code(raw.dtype) if raw is not None else 0, raw.stride(0) if raw is not None else 0, _ptr(raw_bias), _ptr(a_log),
         state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
         _ptr(out), num_seqs, H, KH, N, P, v_cols, chunk, max_chunks, _ptr(ws_state), _ptr(ws_decay), _stream()), "linear_recurrence")
     return out
 
 
-def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor | None, group: int, gate_first: bool, eps: float) -> torch.Tensor:
+GATE_ACTIVATIONS = {"silu": 0, "sigmoid": 1, None: 2}
+
+
+def gated_group_norm(y: torch.Tensor, gate: torch.Tensor | None, weight: torch.Tensor | None, group: int, gate_first: bool, eps: float,
+                     gate_activation: str | None = "silu", out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """Behind a recurrence: y float32 [T, inner], gate [T, inner] (a view, unit inner stride) in the compute type, which is
-    also the result's.  ``gate_first``: u = y silu(gate), u / sqrt(mean(u^2) + eps) * weight over groups of ``group``
-    channels; else y / sqrt(mean(y^2) + eps) * silu(gate) (* weight when given)."""
+    also the result's.  ``gate_first``: u = y act(gate), u / sqrt(mean(u^2) + eps) * weight over groups of ``group``
+    channels; else y / sqrt(mean(y^2) + eps) * act(gate) (* weight when given).  act(z) is z sigmoid(z) ("silu"), sigmoid(z)
+    ("sigmoid"), or 1 (``gate_activation`` None: ``gate`` is None too, and ``out_dtype`` names the result's type)."""
     _on_gpu(y, gate, weight)
     _need(y.dtype == torch.float32 and y.dim() == 2 and y.is_contiguous(), "gated_group_norm y: contiguous float32 [T, inner]")
     T, inner = y.shape
+    _need(gate_activation in GATE_ACTIVATIONS, f"gate_activation: one of {tuple(GATE_ACTIVATIONS)}")
+    if gate is None:
+        _need(gate_activation is None and out_dtype is not None, "without a gate: no gate activation, and the result's type is named")
+        return _group_norm_launch(y, None, 0, out_dtype, weight, group, gate_first, eps, 2)
+    _need(gate_activation is not None, "a gate has an activation")
     _need(gate.shape == (T, inner) and gate.stride(1) == 1, f"gate: [{T}, {inner}] with unit inner stride")
+    return _group_norm_launch(y, gate, gate.stride(0), gate.dtype, weight, group, gate_first, eps, GATE_ACTIVATIONS[gate_activation])
+
+
+def _group_norm_launch(y, gate, gate_stride, dtype, weight, group, gate_first, eps, act):
+    T, inner = y.shape
     _need(group > 0 and inner % group == 0, f"{inner} channels in groups of {group}")
     _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (inner,) and weight.is_contiguous()), f"weight: float32 [{inner}]")
-    out = torch.empty((T, inner), dtype=gate.dtype, device=y.device)
-    sig = [c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]
+    out = torch.empty((T, inner), dtype=dtype, device=y.device)
+    sig = [c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
     _check(_fn("recurrent.hip", "pllm_gated_group_norm", signature=sig)(
-        dtype_code(gate.dtype), _ptr(y), _ptr(gate), gate.stride(0), _ptr(weight), _ptr(out), T, inner, group, 1 if gate_first else 0,
+        dtype_code(dtype), _ptr(y), _ptr(gate), gate_stride, _ptr(weight), _ptr(out), T, inner, group, 1 if gate_first else 0, act,
         c_float(eps), _stream()), "gated_group_norm")
+    return out
+
+
+def silu_to_float(rows: torch.Tensor, cols: int) -> torch.Tensor:
+    """float32 [T, cols]: silu of the first ``cols`` columns of ``rows`` (a view with unit inner stride, either element type):
+    activated operands of a recurrence, which stay in float from here on."""
+    _on_gpu(rows)
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and 0 < cols <= rows.shape[1], f"silu_to_float rows: [T, >= {cols}] with unit inner stride")
+    out = torch.empty((rows.shape[0], cols), dtype=torch.float32, device=rows.device)
+    _check(_fn("recurrent.hip", "pllm_silu_to_float", signature=[c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p])(
+        _ptr(rows), dtype_code(rows.dtype), rows.stride(0), _ptr(out), rows.shape[0], cols, _stream()), "silu_to_float")
+    return out
+
+
+def bounded_forget_gates(rows: torch.Tensor, bias: torch.Tensor | None, lower: torch.Tensor | None, channels: int) -> torch.Tensor:
+    """float32 [3, T, channels] = (q, k, f) from ``rows`` [T, >= 2 channels] laid out [raw_q | raw_f | ...] (a view, either element
+    type): q = silu(raw_q), f = lower + (1 - lower) sigmoid(raw_f + bias), k = 1 - f; ``bias`` and ``lower`` float32 [channels]."""
+    _on_gpu(rows, bias, lower)
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= 2 * channels > 0, f"forget gates' rows: [T, >= {2 * channels}]")
+    for t, what in ((bias, "bias"), (lower, "lower")):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (channels,) and t.is_contiguous()), f"{what}: float32 [{channels}]")
+    out = torch.empty((3, rows.shape[0], channels), dtype=torch.float32, device=rows.device)
+    _check(_fn("recurrent.hip", "pllm_bounded_forget_gates", signature=[c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p])(
+        _ptr(rows), dtype_code(rows.dtype), rows.stride(0), _ptr(bias), _ptr(lower), _ptr(out), rows.shape[0], channels, _stream()),
+        "bounded_forget_gates")
     return out
 
 
@@ -1476,7 +1587,8 @@ def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: to
                  bias: torch.Tensor | None = None, row_index: torch.Tensor | None = None) -> torch.Tensor | None:
     """RMS norms around a float32 residual stream, all in float.  With ``branch`` (float32 rows like the stream, or a
     ``ChoiceSum``: a weighted sum of experts' rows that the kernel forms itself):
-    stream += mult * rms_norm(branch + bias) * w_branch, in place.  Then, when ``out`` or ``out_dtype`` is given, the
+    stream += mult * rms_norm(branch + bias) * w_branch, in place (``w_branch`` None with float32 rows: stream += mult *
+    (branch + bias), the branch as it is: the sum of a pre-norm block).  Then, when ``out`` or ``out_dtype`` is given, the
     rows of the stream as it is now are returned in that type: normed and times ``w_next``, or as they are when
     ``w_next`` is None.  ``out`` may be a view with a row stride of its own (unit inner stride).  Without a branch
     ``row_index`` (int32) picks the rows of the stream; nothing is written to the stream then."""
@@ -1504,8 +1616,8 @@ def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: to
                 out.stride(0) if out is not None else 0, rows, H, _stream()), "rms_sandwich_sum")
             return out
     if branch is not None:
-        _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous() and w_branch is not None,
-              "a branch is contiguous float32 rows like the stream, with its norm's weight")
+        _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous(),
+              "a branch is contiguous float32 rows like the stream (with its norm's weight, or none: it is added as it is)")
         _need(row_index is None, "rows are picked only where no branch is added")
     if row_index is not None:
         _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index must be contiguous int32")
@@ -1518,6 +1630,16 @@ def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: to
                signature=[c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_void_p])(
         dtype_code(out.dtype) if out is not None else F32, _ptr(branch), _ptr(bias), _ptr(w_branch), c_float(mult), _ptr(stream), _ptr(row_index),
         _ptr(w_next), c_float(eps), _ptr(out), out.stride(0) if out is not None else 0, rows, H, _stream()), "rms_sandwich")
+    return out
+
+
+def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float) -> torch.Tensor:
+    """sa * a + sb * b in float, element by element; a and b contiguous, of one shape and type (float32 or the compute type)."""
+    _on_gpu(a, b)
+    _need(a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous(), "scaled_sum: two contiguous tensors of one shape and type")
+    out = torch.empty_like(a)
+    _check(_fn("float_stream.hip", "pllm_scaled_sum", signature=[c_int, c_void_p, c_float, c_void_p, c_float, c_void_p, c_long, c_void_p])(
+        dtype_code(a.dtype), _ptr(a), c_float(sa), _ptr(b), c_float(sb), _ptr(out), a.numel(), _stream()), "scaled_sum")
     return out
 
 
@@ -1584,21 +1706,27 @@ def stream_add(stream: torch.Tensor, branch) -> None:
 
 # ------------------------------------------------------------------------------------------- attention with normed queries and keys
 MAX_PREPARED_HEAD = 256
+VALUE_MODES = {"projected": 0, "normed": 1, "keys": 2}
 
 
 def attn_prepare(proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Tensor | None, state: torch.Tensor | None,
                  state_slots, seq_starts, cu_seqlens, num_seqs: int, positions: torch.Tensor, cos: torch.Tensor | None,
                  sin: torch.Tensor | None, rot: int, interleaved: bool, eps: float, heads: int, kv_heads: int, d: int, dv: int, D: int,
                  dtype: torch.dtype, slot_mapping: torch.Tensor | None, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
-                 qk_norm: bool = True) -> torch.Tensor:
-    """From the float32 sums ``proj`` [T, >= channels] of a q/k/v product (channels = heads d + kv_heads d + kv_heads dv):
+                 qk_norm: bool = True, values: str = "projected") -> torch.Tensor:
+    """``values``: "projected" (the product's value columns as they are), "normed" (each value head divided by its root mean
+    square, ``eps`` inside the root, no weight) or "keys" (the product has no value columns: a value head is its key head
+    as projected, with the bias, before the rotation; dv == d).
+    From the float32 sums ``proj`` [T, >= channels] of a q/k/v product (channels = heads d + kv_heads d + kv_heads dv):
     + ``bias``; a causal convolution over time per channel with ``conv_w`` float32 [channels, taps], whose inputs of
     earlier steps lie in ``state[slot]`` as [taps - 1, channels] and are left there for the next step; rotary encoding
     of the first ``rot`` elements of every q and k head; q and k heads divided by their root mean square (``eps``
     inside the root; not with ``qk_norm`` False); returns q as [T, heads * D] in ``dtype`` (heads padded with zeros to D) and writes k into
     ``k_pages`` [pages, kv_heads, block, D] and v into ``v_pages`` [pages, kv_heads, D, block] at ``slot_mapping``."""
     _on_gpu(proj, bias, conv_w, state, positions, cos, sin, slot_mapping, k_pages, v_pages)
-    channels = (heads + kv_heads) * d + kv_heads * dv
+    _need(values in VALUE_MODES, f"values: one of {tuple(VALUE_MODES)}, got {values!r}")
+    _need(values != "keys" or d == dv, "values that are the keys have the keys' size")
+    channels = (heads + kv_heads) * d + (0 if values == "keys" else kv_heads * dv)
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= channels, f"proj: float32 [T, >= {channels}]")
     T = proj.shape[0]
     _need(0 < d <= D and 0 < dv <= D and D <= MAX_PREPARED_HEAD, f"head sizes {d}, {dv} padded to {D} (at most {MAX_PREPARED_HEAD})")
@@ -1628,12 +1756,12 @@ def attn_prepare(proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Te
         _need(slot_mapping.dtype == torch.int32 and slot_mapping.numel() == T and slot_mapping.is_contiguous(), "slot_mapping: int32 [T]")
     q = torch.empty((T, heads * D), dtype=dtype, device=proj.device)
     sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-           c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
+           c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
     _check(_fn("attention_prepare.hip", "pllm_attn_prepare", signature=sig)(
         dtype_code(dtype), _ptr(proj), proj.stride(0), _ptr(bias), _ptr(conv_w), taps, _ptr(state) if taps > 1 else None,
         state.stride(0) if taps > 1 else 0, _ptr(state_slots) if taps > 1 else None, _ptr(seq_starts) if taps > 1 else None,
         _ptr(cu_seqlens) if taps > 1 else None, num_seqs, _ptr(positions), _ptr(cos) if rot else None, _ptr(sin) if rot else None, rot,
-        int(bool(interleaved)), c_float(eps), int(bool(qk_norm)), heads, kv_heads, d, dv, D, _ptr(q), _ptr(slot_mapping) if write else None,
+        int(bool(interleaved)), c_float(eps), int(bool(qk_norm)), VALUE_MODES[values], heads, kv_heads, d, dv, D, _ptr(q), _ptr(slot_mapping) if write else None,
         _ptr(k_pages) if write else None, _ptr(v_pages) if write else None, bs, T, _stream()), "attn_prepare")
     return q
 

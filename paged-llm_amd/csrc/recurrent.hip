@@ -24,6 +24,9 @@ __device__ __forceinline__ float load_as_f32(const void* p, int dtype, size_t i)
   return dtype == PLLM_F32 ? reinterpret_cast<const float*>(p)[i] : __bfloat162float(reinterpret_cast<const bf16*>(p)[i]);
 }
 __device__ __forceinline__ float silu_f32(float z) { return z / (1.f + expf(-z)); }
+// What a gate's raw value becomes behind a recurrence: z sigmoid(z), sigmoid(z), or 1 (no gate: nothing is read).
+enum { kGateSilu = 0, kGateSigmoid = 1, kGateNone = 2 };
+__device__ __forceinline__ float gate_f32(float z, int act) { return act == kGateSigmoid ? 1.f / (1.f + expf(-z)) : silu_f32(z); }
 
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxTaps = 16;      // most taps of a filter; filters of up to 8 taps take the smaller instance of the kernels
@@ -203,6 +206,9 @@ struct RecurrenceArgs {
   const void* q; const void* k;        // [T, key_heads, N], element type qk_dtype, row stride qk_stride (elements)
   const void* v;                       // [T, heads, P], element type v_dtype, row stride v_stride
   const float* decay;                  // a_t per head: decay[t * decay_stride + h] (decay_stride 0: one number per head)
+  const float* row_decay;              // or a decay per row of S: row_decay[t * row_decay_stride + h * N + n] (then `decay` is null and
+                                       // S_t = diag(row_decay_t) S_(t-1) + k_t (g_t v_t)^T); not together with raw step sizes
+  int row_decay_stride;
   const float* vscale;                 // g_t per head [T, heads], or null for 1
   // or both from raw step sizes [T, heads] (element type raw_dtype, row stride raw_stride):
   //   g_t = softplus(raw + raw_bias[h]) (no clamp),  a_t = exp(-exp(a_log[h]) * g_t)
@@ -238,7 +244,7 @@ enum { kWhole = 0, kChunkState = 1, kChunkOut = 2 };
 
 struct ChunkArgs {
   float* ws_state;      // [chunks][heads][N][P]
-  float* ws_decay;      // [chunks][heads]
+  float* ws_decay;      // [chunks][heads], or [chunks][heads][N] with a decay per row
   int chunk;            // tokens per chunk
   int num_seqs;
 };
@@ -287,7 +293,9 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
   float nl = (with_n && from_state && mine) ? st[(size_t)(n0 + lane) * ld + a.P] : 0.f;
   float decays = 1.f;
   // What a token needs from memory is asked for one token ahead, so that it travels while the token before is computed.
-  struct Fetched { float k, q, x, a, g; };
+  struct Fetched { float k, q, x, a, g, d; };
+  const bool by_row = a.row_decay != nullptr;
+  float decays_l = 1.f;                                      // with a decay per row: the product for row n0 + lane
   auto fetch = [&](int t) {
     Fetched f;
     const size_t row = (size_t)(q_begin + t);
@@ -295,7 +303,12 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     f.k = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
     f.q = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
     f.x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
-    if (a.raw) {
+    f.d = 1.f;
+    if (by_row) {
+      f.d = mine ? a.row_decay[row * a.row_decay_stride + (size_t)head * a.N + n0 + lane] : 1.f;
+      f.a = 1.f;
+      f.g = a.vscale ? a.vscale[row * a.heads + head] : 1.f;
+    } else if (a.raw) {
       f.a = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head);
       f.g = 0.f;
     } else {
@@ -325,6 +338,46 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
       g = cur.g;
     }
     xg = x * g;
+    if (by_row) {
+      const float d_l = cur.d;
+      if (MODE == kChunkState) {
+        const float kw = k_l * decays_l;                  // decays_l: of the tokens behind t in the chunk, for this lane's row
+#pragma unroll
+        for (int i = 0; i < NR; ++i) S[i] = fmaf(row_lane(kw, i), xg, S[i]);
+        if (with_n) nl = fmaf(kw, g, nl);
+        decays_l *= d_l;
+        continue;
+      }
+      float nq = 0.f;
+      if (with_n) {
+        nl = fmaf(k_l, g, d_l * nl);
+        nq = wave_sum(nl * q_l);
+      }
+      float y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        const float kk = row_lane(k_l, i), qq = row_lane(q_l, i), dd = row_lane(d_l, i);
+        S[i] = fmaf(kk, xg, dd * S[i]);
+        y[i & 3] = fmaf(S[i], qq, y[i & 3]);
+      }
+      float total = (y[0] + y[1]) + (y[2] + y[3]);
+      if (waves > 1) {
+        part[t & 1][wv][lane] = total;
+        if (with_n && lane == 0) part_n[t & 1][wv] = nq;
+        __syncthreads();
+        if (wv == 0) {
+          total = part[t & 1][0][lane];
+          for (int w = 1; w < waves; ++w) total += part[t & 1][w][lane];
+          if (with_n) {
+            nq = part_n[t & 1][0];
+            for (int w = 1; w < waves; ++w) nq += part_n[t & 1][w];
+          }
+        }
+      }
+      if (wv == 0 && p_ok) a.out[row * (size_t)(a.heads * ld) + (size_t)head * ld + p] = fmaf(skip, x, total);
+      if (wv == 0 && with_n && lane == 0) a.out[row * (size_t)(a.heads * ld) + (size_t)head * ld + a.P] = nq;
+      continue;
+    }
     if (MODE == kChunkState) {
       const float xw = xg * decays;                       // decays: of the tokens behind t in the chunk
 #pragma unroll
@@ -369,7 +422,9 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
       if (n0 + i < a.N) st[(size_t)(n0 + i) * ld + p] = S[i];
   }
   if (with_n && mine) st[(size_t)(n0 + lane) * ld + a.P] = nl;
-  if (MODE == kChunkState && threadIdx.x == 0 && pb == 0) ca.ws_decay[(size_t)blockIdx.y * a.heads + head] = decays;
+  if (MODE == kChunkState && by_row) {
+    if (pb == 0 && mine) ca.ws_decay[((size_t)blockIdx.y * a.heads + head) * a.N + n0 + lane] = decays_l;
+  } else if (MODE == kChunkState && threadIdx.x == 0 && pb == 0) ca.ws_decay[(size_t)blockIdx.y * a.heads + head] = decays;
 }
 
 // Second pass: per sequence and state element, chunk after chunk:  ws[c] <- the state before chunk c,
@@ -385,13 +440,15 @@ __global__ __launch_bounds__(256) void recurrence_carry_kernel(RecurrenceArgs a,
   for (int s = 0; s < seq; ++s) base += (a.cu_seqlens[s + 1] - a.cu_seqlens[s] + ca.chunk - 1) / ca.chunk;
   const int chunks = (q_len + ca.chunk - 1) / ca.chunk;
   const int head = (int)(idx / per_head);
+  const size_t decay_at = a.row_decay ? (size_t)head * a.N + (idx - (size_t)head * per_head) / a.ld : (size_t)head;
+  const size_t decay_ld = a.row_decay ? (size_t)a.heads * a.N : (size_t)a.heads;
   float* slot = a.state + (size_t)a.state_slots[seq] * a.slot_stride + idx;
   float S = a.seq_starts[seq] > 0 ? *slot : 0.f;
   for (int c = 0; c < chunks; ++c) {
     float* w = ca.ws_state + (size_t)(base + c) * per_seq + idx;
     const float loc = *w;
     *w = S;
-    S = fmaf(ca.ws_decay[(size_t)(base + c) * a.heads + head], S, loc);
+    S = fmaf(ca.ws_decay[(size_t)(base + c) * decay_ld + decay_at], S, loc);
   }
   *slot = S;
 }
@@ -412,17 +469,18 @@ static void launch_recurrence(const RecurrenceArgs& a, const ChunkArgs& ca, dim3
 // over chunks of that many tokens; ws_state holds max_chunks * heads * N * P floats and ws_decay max_chunks * heads, with
 // max_chunks >= sum over the sequences of ceil(q_len / chunk) (total tokens / chunk + num_seqs is enough).
 PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, int qk_stride, const void* v, int v_dtype,
-                                    int v_stride, const float* decay, int decay_stride, const float* vscale, const float* skip,
+                                    int v_stride, const float* decay, int decay_stride, const float* row_decay, int row_decay_stride,
+                                    const float* vscale, const float* skip,
                                     const void* raw, int raw_dtype, int raw_stride, const float* raw_bias, const float* a_log,
                                     float* state, long slot_stride, const int* state_slots, const int* seq_starts,
                                     const int* cu_seqlens, float* out, int num_seqs, int heads, int key_heads, int N, int P,
                                     int v_cols, int chunk, int max_chunks, float* ws_state, float* ws_decay, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
   if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0 || (v_cols != P && v_cols != P - 1)) return -2;
-  if ((raw && (!raw_bias || !a_log)) || (!raw && !decay)) return -2;
+  if ((raw && (!raw_bias || !a_log)) || (!raw && !decay && !row_decay) || (row_decay && (raw || decay || heads != key_heads))) return -2;
   if (chunk < 0 || (chunk > 0 && (max_chunks <= 0 || max_chunks > 65535 || !ws_state || !ws_decay)) || num_seqs > 65535) return -2;
   RecurrenceArgs a;
-  a.q = q; a.k = k; a.v = v; a.decay = decay; a.vscale = vscale; a.skip = skip; a.state = state;
+  a.q = q; a.k = k; a.v = v; a.decay = decay; a.row_decay = row_decay; a.row_decay_stride = row_decay_stride; a.vscale = vscale; a.skip = skip; a.state = state;
   a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
   a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
   a.raw = raw; a.raw_dtype = raw_dtype; a.raw_stride = raw_stride; a.raw_bias = raw_bias; a.a_log = a_log;
@@ -475,7 +533,7 @@ PLLM_API int pllm_step_sizes(int dtype, const void* raw, int raw_stride, const f
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
                                                                int gate_stride, const float* __restrict__ w, T* __restrict__ out,
-                                                               int inner, int group, int gate_first, float eps) {
+                                                               int inner, int group, int gate_first, int gate_act, float eps) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -491,13 +549,13 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __re
     float ss = 0.f;
     for (int i = i0; i < group; i += di) {
       float u = yr[base + i];
-      if (gate_first) u *= silu_f32(to_f32(gr[base + i]));
+      if (gate_first && gate_act != kGateNone) u *= gate_f32(to_f32(gr[base + i]), gate_act);
       ss = fmaf(u, u, ss);
     }
     ss = by_wave ? wave_sum(ss) : block_sum(ss, scratch);
     const float inv = 1.f / sqrtf(ss / (float)group + eps);
     for (int i = i0; i < group; i += di) {
-      const float s = silu_f32(to_f32(gr[base + i]));
+      const float s = gate_act == kGateNone ? 1.f : gate_f32(to_f32(gr[base + i]), gate_act);
       float u = yr[base + i];
       u = gate_first ? (u * s) * inv : (u * inv) * s;
       if (w) u *= w[base + i];
@@ -516,7 +574,7 @@ template <typename T> struct alignas(4 * sizeof(T)) Quad { T v[4]; };
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_regs_kernel(const float* __restrict__ y, const T* __restrict__ gate,
                                                                     int gate_stride, const float* __restrict__ w, T* __restrict__ out,
-                                                                    int inner, int group, int gate_first, float eps) {
+                                                                    int inner, int group, int gate_first, int gate_act, float eps) {
   __shared__ float scratch[4];
   const int row = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -535,11 +593,12 @@ __global__ __launch_bounds__(256) void gated_group_norm_regs_kernel(const float*
       const int at = (j * 64 + lane) * 4;
       if (at < slice) {
         const float4 yv = *reinterpret_cast<const float4*>(yr + base + at);
-        const Quad<T> gv = *reinterpret_cast<const Quad<T>*>(gr + base + at);
+        Quad<T> gv;
+        if (gate_act != kGateNone) gv = *reinterpret_cast<const Quad<T>*>(gr + base + at);
         const float yy[4] = {yv.x, yv.y, yv.z, yv.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          s[j][e] = silu_f32(to_f32(gv.v[e]));
+          s[j][e] = gate_act == kGateNone ? 1.f : gate_f32(to_f32(gv.v[e]), gate_act);
           u[j][e] = gate_first ? yy[e] * s[j][e] : yy[e];
           ss = fmaf(u[j][e], u[j][e], ss);
         }
@@ -578,24 +637,24 @@ static bool group_norm_in_registers(const float* y, const void* gate, int gate_s
 }
 
 PLLM_API int pllm_gated_group_norm(int dtype, const float* y, const void* gate, int gate_stride, const float* w, void* out,
-                                   int num_tokens, int inner, int group, int gate_first, float eps, hipStream_t stream) {
+                                   int num_tokens, int inner, int group, int gate_first, int gate_act, float eps, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
-  if (group <= 0 || inner % group) return -2;
+  if (group <= 0 || inner % group || gate_act < 0 || gate_act > kGateNone || (!gate && gate_act != kGateNone)) return -2;
   dim3 grid(num_tokens), block(256);
   if (dtype == PLLM_F32) {
     if (group_norm_in_registers<float>(y, gate, gate_stride, out, inner, group))
       hipLaunchKernelGGL(gated_group_norm_regs_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
-                         inner, group, gate_first, eps);
+                         inner, group, gate_first, gate_act, eps);
     else
       hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
-                         inner, group, gate_first, eps);
+                         inner, group, gate_first, gate_act, eps);
   } else {
     if (group_norm_in_registers<bf16>(y, gate, gate_stride, out, inner, group))
       hipLaunchKernelGGL(gated_group_norm_regs_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
-                         inner, group, gate_first, eps);
+                         inner, group, gate_first, gate_act, eps);
     else
       hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
-                         inner, group, gate_first, eps);
+                         inner, group, gate_first, gate_act, eps);
   }
   PLLM_RETURN_LAST_ERROR();
 }
@@ -701,5 +760,51 @@ PLLM_API int pllm_mlstm_output(int out_dtype, const float* y, const float* m, co
     hipLaunchKernelGGL(mlstm_output_kernel<float>, grid, block, 0, stream, y, m, gate, gate_dtype, gate_stride, w, (float*)out, heads, P, qscale, eps);
   else
     hipLaunchKernelGGL(mlstm_output_kernel<bf16>, grid, block, 0, stream, y, m, gate, gate_dtype, gate_stride, w, (bf16*)out, heads, P, qscale, eps);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, c] = silu(rows[t, c]) as float for c < cols: the activated q, k and v of a recurrence whose operands stay in float
+// from here on.  rows has a row stride of its own and either element type.
+__global__ __launch_bounds__(256) void silu_to_float_kernel(const void* __restrict__ rows, int dtype, int stride, float* __restrict__ out,
+                                                            int cols, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / cols, c = i - t * cols;
+  out[i] = silu_f32(load_as_f32(rows, dtype, t * stride + c));
+}
+
+PLLM_API int pllm_silu_to_float(const void* rows, int dtype, int stride, float* out, int num_tokens, int cols, hipStream_t stream) {
+  if (num_tokens <= 0 || cols <= 0) return 0;
+  const size_t total = (size_t)num_tokens * cols;
+  hipLaunchKernelGGL(silu_to_float_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, rows, dtype, stride, out, cols, total);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// A forget gate with a lower bound per channel, whose complement is the key (a recurrence without a key product):
+//   f = lower + (1 - lower) * sigmoid(raw_f + bias),   k = 1 - f,   q = silu(raw_q),
+// from rows [T, >= 2 channels] laid out [raw_q | raw_f | ...]; out float [3][T][channels] = q, k, f.
+__global__ __launch_bounds__(256) void bounded_forget_gates_kernel(const void* __restrict__ rows, int dtype, int stride,
+                                                                   const float* __restrict__ bias, const float* __restrict__ lower,
+                                                                   float* __restrict__ out, int channels, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / channels, c = i - t * channels;
+  const float zq = load_as_f32(rows, dtype, t * stride + c);
+  const float zf = load_as_f32(rows, dtype, t * stride + channels + c) + (bias ? bias[c] : 0.f);
+  const float lo = lower ? lower[c] : 0.f;
+  const float sg = 1.f / (1.f + expf(-zf));
+  const float f = lo + (1.f - lo) * sg;
+  out[i] = silu_f32(zq);
+  out[total + i] = 1.f - f;
+  out[2 * total + i] = f;
+}
+
+PLLM_API int pllm_bounded_forget_gates(const void* rows, int dtype, int stride, const float* bias, const float* lower, float* out,
+                                       int num_tokens, int channels, hipStream_t stream) {
+  if (num_tokens <= 0 || channels <= 0) return 0;
+  const size_t total = (size_t)num_tokens * channels;
+  hipLaunchKernelGGL(bounded_forget_gates_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, rows, dtype, stride, bias,
+                     lower, out, channels, total);
   PLLM_RETURN_LAST_ERROR();
 }

@@ -51,7 +51,7 @@ def build_runtime(model: DecoderModel, block_size: int, num_pages: int | dict, n
     """(CacheManager, KVCacheStorage, ModelRunner) for a model: one page pool per cache group,
     one state slot pool when a mixer keeps per-request state."""
     groups = model.cache_groups()
-    specs = [GroupSpec(name, g.spec.kind, g.spec.window) for name, g in groups.items()]
+    specs = [GroupSpec(name, g.spec.kind, g.spec.window, g.spec.keep_first) for name, g in groups.items()]
     uses_state = bool(model.state_specs())
     manager = CacheManager(specs, num_pages, block_size, enable_prefix_caching,
                            num_state_slots=num_state_slots if uses_state else 0)

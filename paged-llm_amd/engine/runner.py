@@ -179,6 +179,8 @@ class ModelRunner:
                 else:
                     row = np.asarray(table[:need], dtype=np.int64)
                     live = row[first_key // bs:]
+                    if cs.keep_first:                                  # the pages of the kept first positions are read as well
+                        live = np.concatenate([row[:min(-(-cs.keep_first // bs), first_key // bs)], live])
                     if live.size and (live.min() < 0 or live.max() >= num_pages):
                         raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
                     shown = np.where(row == NO_PAGE, 0, row).astype(np.int32)
@@ -377,6 +379,8 @@ class ModelRunner:
                 row = np.asarray(table[:n], dtype=np.int64)
                 first_key = first_visible_key(cs.kind, cs.window, e.start)
                 live = row[first_key // bs:]
+                if cs.keep_first:
+                    live = np.concatenate([row[:min(-(-cs.keep_first // bs), first_key // bs)], live])
                 if live.size and (live.min() < 0 or live.max() >= num_pages):
                     raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
                 tables[s, :n] = np.where(row == NO_PAGE, 0, row)

@@ -13,6 +13,8 @@ from ..parts.spec import ModelSpec, WeightSpec
 
 
 class DecoderModel:
+    EMBEDDING_STATE = "embedding"       # key of the embedding's per-request state among the states of the schedule's steps
+
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device, max_positions: int | None = None):
         self.spec = spec
         self.dtype = dtype
@@ -58,6 +60,8 @@ class DecoderModel:
             own = name_under(prefix, name)
             if own is not None and own in part.weight_specs():
                 return part.assign(own, tensor)
+            if "/" + name in part.weight_specs():             # a tensor that the part names outside its prefix
+                return part.assign("/" + name, tensor)
         for layer, block in zip(s.layers, self.blocks):
             own = name_under(layer.name, name)
             if own:
@@ -93,6 +97,8 @@ class DecoderModel:
     def state_specs(self) -> dict[int, object]:
         """Schedule step -> StateSpec for mixers with per-request state of fixed size."""
         out = {}
+        if getattr(self.embedding, "state_spec", None) is not None and self.embedding.state_spec() is not None:
+            out[self.EMBEDDING_STATE] = self.embedding.state_spec()       # (an embedding that looks at the token before)
         for pos, step in enumerate(self.spec.schedule):
             ss = self.blocks[step.layer].state_spec()
             if ss is not None:
@@ -117,23 +123,31 @@ class DecoderModel:
         """Float logits [n, vocab] at ctx.logits_index (empty tensor when nothing is wanted;
         the layers still run to fill the cache)."""
         assert self._ready, "weights not loaded"
-        x = self.embedding.forward(ctx.input_ids)
+        stateful_embedding = hasattr(self.embedding, "forward_step")
+        x = (self.embedding.forward_step(ctx, states.get(self.EMBEDDING_STATE)) if stateful_embedding
+             else self.embedding.forward(ctx.input_ids))
         delta = None
         schedule = self.spec.schedule
         # the embedding's output for the stream operations: a tensor of its own where the layers add to the stream in place
         x0 = None
         if self.stream_ops:
-            x0 = self.embedding.forward(ctx.input_ids) if getattr(self.embedding, "float_stream", False) else x
+            if stateful_embedding:
+                x0 = self.embedding.forward_step(ctx, states.get(self.EMBEDDING_STATE), again=True)
+            else:
+                x0 = self.embedding.forward(ctx.input_ids) if getattr(self.embedding, "float_stream", False) else x
         last_takes_partial = bool(getattr(self.final_norm, "accepts_partial_sums", False))
         for pos, step in enumerate(schedule):
             block = self.blocks[step.layer]
-            if step.entry is not None:
-                if delta is not None:
-                    raise RuntimeError("a stream operation takes the stream with every sum done")
-                x = self.stream_ops[step.entry].forward(x, x0, ctx)
+            if step.entry is not None and delta is not None:
+                raise RuntimeError("a stream operation takes the stream with every sum done")
             # the norm that reads the stream next, for a block that can compute its rows while it forms the stream's last sum
             following = schedule[pos + 1] if pos + 1 < len(schedule) else None
             ctx.next_entry_norm = (self.blocks[following.layer].entry_norm() if following is not None and following.entry is None else None)
+            if step.entry is not None:
+                # the stream operation in front of this layer may norm for the layer in the kernel that forms its sum
+                ctx.next_entry_norm, after_op = block.entry_norm(), ctx.next_entry_norm
+                x = self.stream_ops[step.entry].forward(x, x0, ctx)
+                ctx.next_entry_norm = after_op
             cache = None
             if block.cache_spec() is not None:
                 owner = pos if step.cache_from is None else step.cache_from

@@ -29,7 +29,10 @@ BLOCK = "block"       # in the shape of a page tensor: the dimension that holds 
 
 def tensor_name(prefix: str, name: str) -> str:
     """The checkpoint name of a part's tensor: the part's prefix, a dot, the tensor's own name; a tensor whose own name
-    is empty bears the prefix itself (a norm's weight stored as "final.norm" beside its bias "final.norm.b")."""
+    is empty bears the prefix itself (a norm's weight stored as "final.norm" beside its bias "final.norm.b"); an own name
+    that starts with "/" is the checkpoint name itself, outside the prefix (a second table of an embedding stored beside it)."""
+    if name.startswith("/"):
+        return name[1:]
     return f"{prefix}.{name}" if name else prefix
 
 
@@ -74,16 +77,19 @@ class CacheSpec:
                               # "chunk": only the positions of the newest block of `window` positions (blocks counted from 0)
     tensors: tuple            # of PageTensor
     window: int = 0           # > 0 for the kinds "window" and "chunk"
+    keep_first: int = 0       # kind "window": the sequence's first positions stay visible to every later query (their pages are kept)
 
     def __post_init__(self):
         if self.kind not in ("full", "window", "chunk") or (self.kind != "full") != (self.window > 0):
             raise ValueError(f"cache kind {self.kind!r} with window {self.window}: \"full\", or \"window\" / \"chunk\" with a size > 0")
+        if self.keep_first < 0 or (self.keep_first > 0 and self.kind != "window"):
+            raise ValueError(f"first positions are kept beside a sliding window only; got {self.keep_first} with kind {self.kind!r}")
         names = [t.name for t in self.tensors]
         if not names or len(set(names)) != len(names):
             raise ValueError(f"a cache spec names at least one page tensor, each once; got {names}")
 
     def group_name(self) -> str:
-        base = f"{self.kind}{self.window if self.kind != 'full' else ''}"
+        base = f"{self.kind}{self.window if self.kind != 'full' else ''}" + (f"keep{self.keep_first}" if self.keep_first else "")
         def one(t):
             dims = "x".join("B" if d == BLOCK else str(d) for d in t.shape)
             return f"{t.name}{dims}" + (f":{str(t.dtype).split('.')[-1]}" if t.dtype is not None else "")

@@ -193,9 +193,11 @@ class FloatPreNormBlock(Block):
     def _entry_rows(self, x, ctx):
         """norm_a(x) in the compute type: what the kernel that last wrote x left for this norm, or computed now."""
         norm = self.parts["mixer_norm"]
-        held = ctx.launch_cache.get(self._ROWS)
-        if held is not None and held[0] is x and held[1] is norm:
-            return held[2]
+        for key in (self._ROWS, "stream_entry_rows"):        # (the second: left by a stream operation in front of this layer)
+            held = ctx.launch_cache.get(key)
+            if held is not None and held[0] is x and held[1] is norm:
+                ctx.launch_cache[key] = None
+                return held[2]
         return norm.forward(x)
 
     def forward(self, x, delta, ctx, cache, state):

@@ -42,6 +42,56 @@ class TokenEmbedding(Part):
         return ops.embed_gather(ids, self.table)
 
 
+class HashedBigramEmbedding(Part):
+    """A token embedding to which a row of a second table is added, chosen by a hash of the token before and the token
+    itself:  x = table[token] * scale + pairs[(previous * mul_prev + token * mul_cur) mod buckets], and the second table's
+    last row (number ``buckets``) for a sequence's first token.  The rows leave as float32 (the start of a residual stream
+    summed in float).  The token before a step's first token is per-request state: one int32 per slot, left there by the
+    step before (``state_spec``); a request at position 0 has none, whatever its slot holds.
+
+    params: ``vocab_size``, ``scale``, ``buckets``, ``mul_prev``, ``mul_cur``; ``tensor_name`` (the token table's own name
+    under the part's prefix; "" is the prefix itself) and ``pairs_name`` (the second table's; "/name" is a name outside the prefix)."""
+    float_stream = True
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.vocab = int(params["vocab_size"])
+        self.hidden = env.hidden_size
+        self.scale = float(params.get("scale") or 1.0)
+        self.buckets, self.mul_prev, self.mul_cur = int(params["buckets"]), int(params["mul_prev"]), int(params["mul_cur"])
+        if self.buckets <= 0:
+            raise ValueError(f"a bigram table needs a positive number of buckets, got {self.buckets}")
+        self.tensor_name = params.get("tensor_name", "weight")
+        self.pairs_name = params.get("pairs_name", "pairs")
+        self.dtype, self.device = env.dtype, env.device
+        self.table: torch.Tensor | None = None
+        self.pairs: torch.Tensor | None = None
+        self._rows = None            # the bigram rows of the step under way, for a second gather of the same step
+
+    def weight_specs(self):
+        return {self.tensor_name: WeightSpec((self.vocab, self.hidden), role="table"),
+                self.pairs_name: WeightSpec((self.buckets + 1, self.hidden), role="table")}
+
+    def assign(self, name, tensor):
+        t = tensor.to(device=self.device, dtype=self.dtype).contiguous()
+        if name == self.tensor_name:
+            self.table = t
+        elif name == self.pairs_name:
+            self.pairs = t
+        else:
+            raise KeyError(name)
+
+    def state_spec(self):
+        from .base import StateSpec
+        return StateSpec((1,), torch.int32)
+
+    def forward_step(self, ctx, state: torch.Tensor, again: bool = False) -> torch.Tensor:
+        """The step's rows; ``again``: once more for the same step (the state has moved already)."""
+        if not again:
+            self._rows = torch.empty_like(ctx.input_ids)
+        return ops.embed_bigram(ctx.input_ids, self.table, self.pairs, self.scale, self.buckets, self.mul_prev, self.mul_cur, state,
+                                ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs, self._rows, move_state=not again)
+
+
 class LMHead(Part):
     def __init__(self, params: dict, env: BuildEnv):
         self.vocab = int(params["vocab_size"])
@@ -74,4 +124,5 @@ class LMHead(Part):
 
 
 register_embedding("token_embedding", TokenEmbedding)
+register_embedding("hashed_bigram_embedding", HashedBigramEmbedding)
 register_head("lm_head", LMHead)

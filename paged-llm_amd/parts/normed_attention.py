@@ -32,9 +32,15 @@ class NormedAttention(Mixer):
     rotary spec or None), ``mask`` ("full", "window" or "chunk") with ``mask_size``, ``conv`` (taps of the convolution
     over time; 0: none), ``bias`` (q, k, v and the output product have biases), ``sinks`` (a logit per head in the
     softmax's sum), ``head_gate`` (a gate per head from the mixer's input), ``qk_norm`` (default True; False: q and k go
-    to the scores as they are rotated), ``score_cap`` c > 0 (the scaled product x becomes c tanh(x / c); default none).  Tensors (under the part's prefix): ``q``,
+    to the scores as they are rotated), ``score_cap`` c > 0 (the scaled product x becomes c tanh(x / c); default none);
+    ``output_bias`` (default: as ``bias``; False: the projections have biases, the output product has none);
+    ``values``: "projected" (default), "normed" (every value head divided by its root mean square, ``eps`` inside the root, no
+    weight, and cached so) or "keys" (there is no value product: a value head is its key head as projected, before the
+    rotation; the two sizes are equal); ``keep_first`` (with a window: the sequence's first positions that every later query
+    still sees, at their own positions); ``weighting``: "softmax" (default) or "sigmoid" (a visible key weighs
+    sigmoid(score + ``pb``[head]), not normalised over the keys).  Tensors (under the part's prefix): ``q``,
     ``k``, ``v``, ``o``; ``q.b``, ``k.b``, ``v.b``, ``o.b``; ``q.conv``, ``k.conv``, ``v.conv`` [channels, taps];
-    ``sink`` [heads]; ``g`` [heads, width]."""
+    ``sink`` [heads]; ``g`` [heads, width]; ``pb`` [heads]."""
     graph_capturable = True
     graph_capturable_prompts = True
 
@@ -48,6 +54,18 @@ class NormedAttention(Mixer):
         self.taps = max(1, int(params.get("conv") or 1))
         self.bias, self.has_sinks, self.head_gate = bool(params.get("bias")), bool(params.get("sinks")), bool(params.get("head_gate"))
         self.qk_norm, self.score_cap = bool(params.get("qk_norm", True)), float(params.get("score_cap") or 0.0)
+        self.out_bias = bool(params.get("output_bias", self.bias))
+        self.values = params.get("values") or "projected"
+        self.keep_first = int(params.get("keep_first") or 0)
+        self.weighting = params.get("weighting") or "softmax"
+        if self.values not in ops.VALUE_MODES or self.weighting not in ("softmax", "sigmoid"):
+            raise ValueError(f"values {self.values!r}: one of {tuple(ops.VALUE_MODES)}; weighting {self.weighting!r}: softmax or sigmoid")
+        if self.values == "keys" and self.d != self.dv:
+            raise ValueError(f"values that are the keys have the keys' size: {self.dv} against {self.d}")
+        if self.keep_first < 0 or (self.keep_first > 0 and self.mask != "window"):
+            raise ValueError("first positions are kept beside a sliding window only")
+        if self.weighting == "sigmoid" and self.has_sinks:
+            raise ValueError("a sink is a term of a softmax's sum: there is none under sigmoid weights")
         if self.score_cap < 0.0:
             raise ValueError(f"a cap of the scores is positive (or 0 for none), got {self.score_cap}")
         if self.heads % self.kv_heads:
@@ -62,23 +80,30 @@ class NormedAttention(Mixer):
         pos = params.get("position")
         self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
         self.rot = (self.position.rotary_dim or self.d) if self.position is not None else 0
-        self.channels = (self.heads + self.kv_heads) * self.d + self.kv_heads * self.dv
+        self.channels = (self.heads + self.kv_heads) * self.d + (0 if self.values == "keys" else self.kv_heads * self.dv)
         self.dtype, self.device = env.dtype, env.device
         # the mask as the attention kernels take it: > 0 a window, < 0 blocks of that many positions
         self.window = self.mask_size if self.mask == "window" else (-self.mask_size if self.mask == "chunk" else 0)
         self._w: dict = {}
-        self.w_in = self.w_o = self.b_in = self.output_bias = self.conv_w = self.terms = None
+        self.w_in = self.w_o = self.b_in = self.output_bias = self.conv_w = self.terms = self.weights = None
 
     # ---- weights
     def weight_specs(self):
         q, k, v = self.heads * self.d, self.kv_heads * self.d, self.kv_heads * self.dv
-        specs = {"q": WeightSpec((q, self.hidden)), "k": WeightSpec((k, self.hidden)), "v": WeightSpec((v, self.hidden)),
-                 "o": WeightSpec((self.hidden, self.heads * self.dv))}
+        own_values = self.values != "keys"
+        specs = {"q": WeightSpec((q, self.hidden)), "k": WeightSpec((k, self.hidden)), "o": WeightSpec((self.hidden, self.heads * self.dv))}
+        if own_values:
+            specs["v"] = WeightSpec((v, self.hidden))
         if self.bias:
-            specs.update({"q.b": WeightSpec((q,), role="vector"), "k.b": WeightSpec((k,), role="vector"), "v.b": WeightSpec((v,), role="vector"),
-                          "o.b": WeightSpec((self.hidden,), role="vector")})
+            specs.update({"q.b": WeightSpec((q,), role="vector"), "k.b": WeightSpec((k,), role="vector")})
+            if own_values:
+                specs["v.b"] = WeightSpec((v,), role="vector")
+        if self.out_bias:
+            specs["o.b"] = WeightSpec((self.hidden,), role="vector")
         if self.has_conv:
-            specs.update({f"{n}.conv": WeightSpec((c, self.taps), role="vector") for n, c in (("q", q), ("k", k), ("v", v))})
+            specs.update({f"{n}.conv": WeightSpec((c, self.taps), role="vector") for n, c in (("q", q), ("k", k), ("v", v))[:3 if own_values else 2]})
+        if self.weighting == "sigmoid":
+            specs["pb"] = WeightSpec((self.heads,), role="vector")
         if self.has_sinks:
             specs["sink"] = WeightSpec((self.heads,), role="vector")
         if self.head_gate:
@@ -93,20 +118,24 @@ class NormedAttention(Mixer):
 
     def finalize(self):
         w = self._w
-        self.w_in = Weight(torch.cat([w.pop(n) for n in ("q", "k", "v") + (("g",) if self.head_gate else ())], dim=0).contiguous())
+        qkv = ("q", "k", "v") if self.values != "keys" else ("q", "k")
+        self.w_in = Weight(torch.cat([w.pop(n) for n in qkv + (("g",) if self.head_gate else ())], dim=0).contiguous())
         self.w_o = Weight(w.pop("o"))
         if self.bias:
-            self.b_in = torch.cat([w.pop(n) for n in ("q.b", "k.b", "v.b")]).contiguous()
-            self.output_bias = w.pop("o.b")           # added by whoever norms the mixer's float output (the block's kernel)
+            self.b_in = torch.cat([w.pop(n + ".b") for n in qkv]).contiguous()
+        if self.out_bias:
+            self.output_bias = w.pop("o.b")           # added by whoever norms the mixer's float output (the block's kernel), or by the product
         if self.has_conv:
-            self.conv_w = torch.cat([w.pop(n) for n in ("q.conv", "k.conv", "v.conv")], dim=0).contiguous()
+            self.conv_w = torch.cat([w.pop(n + ".conv") for n in qkv], dim=0).contiguous()
+        if self.keep_first or self.weighting == "sigmoid":
+            self.weights = ops.KeyWeights(self.keep_first, self.weighting == "sigmoid", w.pop("pb") if self.weighting == "sigmoid" else None)
         terms = ops.ScoreTerms(self.score_cap, None, w.pop("sink") if self.has_sinks else None)
         self.terms = terms if terms.any() else None
 
     # ---- what it keeps
     def cache_spec(self):
         G, D = self.kv_heads, self.D
-        return CacheSpec(self.mask, (PageTensor("k", (G, BLOCK, D)), PageTensor("v", (G, D, BLOCK))), self.mask_size)
+        return CacheSpec(self.mask, (PageTensor("k", (G, BLOCK, D)), PageTensor("v", (G, D, BLOCK))), self.mask_size, self.keep_first)
 
     def state_spec(self):
         return StateSpec(((self.taps - 1) * self.channels,), torch.float32) if self.taps > 1 else None
@@ -129,9 +158,9 @@ class NormedAttention(Mixer):
         q = ops.attn_prepare(proj, self.b_in, self.conv_w, state, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
                              ctx.positions, pe.cos if pe is not None else None, pe.sin if pe is not None else None, self.rot,
                              bool(pe.interleaved) if pe is not None else False, self.eps, H, G, self.d, self.dv, D, self.dtype,
-                             view.slot_mapping, k_pages, v_pages, qk_norm=self.qk_norm)
+                             view.slot_mapping, k_pages, v_pages, qk_norm=self.qk_norm, values=self.values)
         o = ops.paged_attention(q, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k, H, G, D, self.scale,
-                                self.window, ctx, terms=self.terms)
+                                self.window, ctx, terms=self.terms, weights=self.weights)
         if self.head_gate or D != self.dv:
             o = ops.gate_heads(o, proj[:, self.channels:self.channels + H] if self.head_gate else None, H, self.dv, D)
         out_dtype = torch.float32 if getattr(ctx, "float_branch", False) else None

@@ -17,6 +17,13 @@ Both are the same recurrence per head, S_t = a_t S_(t-1) + k_t (g_t v_t)^T, y_t 
   column of S; y_t is divided by max(|n_t . q_t|, exp(-m_t)), then by its root mean square per head, times a weight,
   times the sigmoid of the output gate, the output product.
 
+* ``lightning`` (linear attention with a constant decay per head): q, k and v pass SiLU and stay in float from there; no
+  positions, no scale; behind the recurrence all heads' outputs are divided by their common root mean square, times a weight,
+  times the sigmoid of a gate, the output product.
+* ``hgrn2`` (a gated linear recurrence without a key product): the forget gate f, bounded below per channel, decays the
+  rows of S one by one, S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T; q passes SiLU; behind it each head's output is divided by
+  its root mean square, times a weight that the heads share, the output product.
+
 What enters the recurrence (step sizes, decays, rotated keys and queries, the state) is float whatever the compute type;
 the products, the convolution and the activations run in the compute type.  A request's state is zero at its first
 token (``ctx.seq_starts == 0``), whatever its slot held before.
@@ -210,6 +217,98 @@ class MLstmMixer(_StatefulMixer):
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
 
+class LightningMixer(_StatefulMixer):
+    """Linear attention with one constant decay per head:  q = silu(W_q h), k = silu(W_k h), v = silu(W_v h),
+    S_t = decay_h S_(t-1) + k_t v_t^T,  o_t = S_t^T q_t  (no scale, no positions); then all heads' outputs side by side are
+    divided by their root mean square, times ``norm``, times sigmoid(W_g h), and projected.  The activated q, k, v, the state
+    and the norm are float whatever the compute type.
+
+    params: ``heads``, ``key_dim`` (N), ``head_dim`` (P), ``decay`` (one number per head), ``eps``.  Tensors ``q``, ``k`` [heads N,
+    width], ``v``, ``g`` [heads P, width], ``norm`` [heads P], ``o`` [width, heads P]."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.heads, self.N, self.P = int(params["heads"]), int(params["key_dim"]), int(params["head_dim"])
+        self.eps = float(params["eps"])
+        decay = [float(d) for d in params["decay"]]
+        if len(decay) != self.heads:
+            raise ValueError(f"{len(decay)} decays for {self.heads} heads")
+        self.dtype, self.device = env.dtype, env.device
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=self.device)
+        self._w: dict = {}
+        self.w_in = self.w_o = None
+
+    def weight_specs(self):
+        qk, vg = self.heads * self.N, self.heads * self.P
+        return {"q": WeightSpec((qk, self.hidden)), "k": WeightSpec((qk, self.hidden)), "v": WeightSpec((vg, self.hidden)),
+                "g": WeightSpec((vg, self.hidden)), "norm": WeightSpec((vg,), role="vector", init="ones"), "o": WeightSpec((self.hidden, vg))}
+
+    def finalize(self):
+        self.w_in = Weight(torch.cat([self._w.pop(n) for n in ("q", "k", "v", "g")], dim=0).contiguous())
+        self.w_o = Weight(self._w.pop("o"))
+
+    def state_spec(self):
+        return StateSpec((self.heads * self.N * self.P,), torch.float32)
+
+    def forward(self, h, ctx, cache, state):
+        H, N, P = self.heads, self.N, self.P
+        rows = linear(h, self.w_in)
+        qk, vg = H * N, H * P
+        acts = ops.silu_to_float(rows, 2 * qk + vg)
+        q, k = acts[:, :qk].unflatten(1, (H, N)), acts[:, qk:2 * qk].unflatten(1, (H, N))
+        v = acts[:, 2 * qk:].unflatten(1, (H, P))
+        y = ops.linear_recurrence(q, k, v, self.decay, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
+                                  max_q_len=ctx.max_q_len)
+        u = ops.gated_group_norm(y, rows[:, 2 * qk + vg:], self._w["norm"], vg, False, self.eps, gate_activation="sigmoid")
+        return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
+
+
+class Hgrn2Mixer(_StatefulMixer):
+    """A gated linear recurrence whose forget gate also decides what is written:  q = silu(W_q h), v = W_v h,
+    f = l + (1 - l) sigmoid(W_f h + b_f) per head and channel with a stored lower bound l,
+    S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T,  o_t = S_t^T q_t;  then each head's o divided by its root mean square, times
+    ``norm`` (one weight over a head's channels, shared by the heads), the output product.  Gates, decays, the state and the
+    norm are float whatever the compute type (the input product leaves float sums).
+
+    params: ``heads``, ``key_dim`` (N), ``head_dim`` (P), ``eps``.  Tensors ``q``, ``f`` [heads N, width], ``f.b``, ``lower`` [heads N],
+    ``v`` [heads P, width], ``norm`` [P], ``o`` [width, heads P]."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.heads, self.N, self.P = int(params["heads"]), int(params["key_dim"]), int(params["head_dim"])
+        self.eps = float(params["eps"])
+        self.dtype, self.device = env.dtype, env.device
+        self._w: dict = {}
+        self.w_in = self.w_o = self.norm_w = None
+
+    def weight_specs(self):
+        qf, v = self.heads * self.N, self.heads * self.P
+        return {"q": WeightSpec((qf, self.hidden)), "f": WeightSpec((qf, self.hidden)), "f.b": WeightSpec((qf,), role="vector"),
+                "lower": WeightSpec((qf,), role="vector", init="zeros"), "v": WeightSpec((v, self.hidden)),
+                "norm": WeightSpec((self.P,), role="vector", init="ones"), "o": WeightSpec((self.hidden, v))}
+
+    def finalize(self):
+        self.w_in = Weight(torch.cat([self._w.pop(n) for n in ("q", "f", "v")], dim=0).contiguous())
+        self.w_o = Weight(self._w.pop("o"))
+        self.norm_w = self._w.pop("norm").repeat(self.heads).contiguous()       # the heads share one weight
+
+    def state_spec(self):
+        return StateSpec((self.heads * self.N * self.P,), torch.float32)
+
+    def forward(self, h, ctx, cache, state):
+        H, N, P = self.heads, self.N, self.P
+        rows = linear(h, self.w_in, out_dtype=torch.float32)
+        qkf = ops.bounded_forget_gates(rows, self._w["f.b"], self._w["lower"], H * N)
+        q, k, f = (qkf[i].unflatten(1, (H, N)) for i in range(3))
+        v = rows[:, 2 * H * N:].unflatten(1, (H, P))
+        y = ops.linear_recurrence(q, k, v, None, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
+                                  max_q_len=ctx.max_q_len, row_decay=f)
+        u = ops.gated_group_norm(y, None, self.norm_w, P, False, self.eps, gate_activation=None, out_dtype=self.dtype)
+        return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
+
+
+register_mixer("lightning", LightningMixer)
+register_mixer("hgrn2", Hgrn2Mixer)
 register_mixer("mamba2", Mamba2Mixer)
 register_mixer("retention", RetentionMixer)
 register_mixer("mlstm", MLstmMixer)

@@ -1,7 +1,7 @@
 """Rotary position encoding: float tables of cos and sin per position.
 
 inv_freq[i] = 1 / theta^(2i/r) over the r rotated elements of a head; optional "llama3" rescale of the
-low frequencies; angle[p, i] = p * inv_freq[i] in float (pagedllm/model/llama.py:86-128).  The tables
+low frequencies, or a "yarn" rescale (frequencies blended by pair index, both tables times 0.1 ln(factor) + 1); angle[p, i] = p * inv_freq[i] in float (pagedllm/model/llama.py:86-128).  The tables
 hold r/2 columns (the reference's cat[freqs, freqs] repeats them).  The rotation itself is done by the
 mixer's kernel, fused with the cache write; this part says how: ``rotary_dim`` = r (default: the whole
 head, as in the reference) and ``interleaved`` (pairs (2i, 2i+1) instead of the reference's (i, i + r/2)).
@@ -32,6 +32,22 @@ def llama3_rescale(inv_freq: torch.Tensor, factor: float, low_freq_factor: float
     return torch.where(middle, blended, out)
 
 
+def yarn_rescale(inv_freq: torch.Tensor, base: float, factor: float, original: float, fast: float, slow: float) -> torch.Tensor:
+    """Frequencies blended by the index of their pair: with idx(t) = r ln(original / (2 pi t)) / (2 ln base) the (real) index
+    of the pair that makes t turns over ``original`` positions, lo = max(floor(idx(fast)), 0), hi = min(ceil(idx(slow)), r - 1)
+    and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * ramp_i + f_i (1 - ramp_i):
+    the pairs below lo as they are, those above hi slowed by the factor."""
+    r = 2 * inv_freq.numel()
+
+    def index_of(turns: float) -> float:
+        return r * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo = max(math.floor(index_of(fast)), 0)
+    hi = min(math.ceil(index_of(slow)), r - 1)
+    ramp = ((torch.arange(inv_freq.numel(), dtype=inv_freq.dtype) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return inv_freq / factor * ramp + inv_freq * (1.0 - ramp)
+
+
 class RotaryEncoding(PositionEncoding):
     def __init__(self, params: dict, env: BuildEnv):
         self.head_dim = int(params["head_dim"])
@@ -47,15 +63,29 @@ class RotaryEncoding(PositionEncoding):
                              f"size {self.head_dim}, got {self.rotary_dim}")
         if self.scaling:
             kind = self.scaling.get("rope_type", self.scaling.get("type"))
-            if kind != "llama3":
-                raise NotImplementedError(f"rope_type={kind!r} not supported (default and llama3 only)")
+            if kind not in ("llama3", "yarn"):
+                raise NotImplementedError(f"rope_type={kind!r} not supported (default, llama3 and yarn only)")
         self.device = env.device
         self.cos: torch.Tensor | None = None
         self.sin: torch.Tensor | None = None
         self.num_positions = 0
 
+    def _yarn(self) -> dict | None:
+        s = self.scaling
+        return s if s and s.get("rope_type", s.get("type")) == "yarn" else None
+
+    def table_factor(self) -> float:
+        """What both tables are multiplied by: 0.1 ln(factor) + 1 under the "yarn" rescaling, else 1."""
+        s = self._yarn()
+        return 0.1 * math.log(float(s["factor"])) + 1.0 if s else 1.0
+
     def inverse_frequencies(self) -> torch.Tensor:
         d = self.rotary_dim
+        if self._yarn():
+            # (always formed in double precision and rounded once)
+            s = self._yarn()
+            inv_freq = torch.tensor([self.theta ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64)
+            return yarn_rescale(inv_freq, self.theta, float(s["factor"]), float(s["original"]), float(s["fast"]), float(s["slow"])).to(torch.float32)
         if self.exact_frequencies:
             inv_freq = torch.tensor([self.theta ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64)
             if self.scaling:
@@ -76,8 +106,9 @@ class RotaryEncoding(PositionEncoding):
             return
         t = torch.arange(max_positions, dtype=torch.float32)
         angles = torch.outer(t, self.inverse_frequencies())          # [P, rotary_dim/2], float
-        self.cos = angles.cos().to(self.device).contiguous()
-        self.sin = angles.sin().to(self.device).contiguous()
+        mag = self.table_factor()
+        self.cos = (angles.cos() * mag if mag != 1.0 else angles.cos()).to(self.device).contiguous()
+        self.sin = (angles.sin() * mag if mag != 1.0 else angles.sin()).to(self.device).contiguous()
         self.num_positions = max_positions
 
 

@@ -46,3 +46,28 @@ class ConcatProjection(StreamOp):
 
 
 register_stream_op("concat_projection", ConcatProjection)
+
+
+class AddEmbedding(StreamOp):
+    """x <- x + x0: the embedding's output added to the stream, in float and in place (x0 itself is never written to).  When
+    the layer behind it norms with a norm that can follow a sum in its kernel (``ctx.next_entry_norm`` with ``sum_then``), that
+    norm's rows of the new stream come from the same kernel and travel beside the stream in ``ctx.launch_cache``
+    (``ENTRY_ROWS``: (stream, norm, rows)), where a block over a float stream looks for them."""
+    ENTRY_ROWS = "stream_entry_rows"
+
+    def __init__(self, params: dict, env: BuildEnv):
+        pass
+
+    def forward(self, x, x0, ctx):
+        if x.dtype != torch.float32 or x0.dtype != torch.float32 or x0 is x:
+            raise RuntimeError("the embedding's output is added to a float stream, and is a tensor of its own")
+        norm = getattr(ctx, "next_entry_norm", None)
+        if norm is not None and hasattr(norm, "sum_then"):
+            ctx.launch_cache[self.ENTRY_ROWS] = (x, norm, norm.sum_then(x, x0))
+        else:
+            ops.stream_add(x, x0)
+            ctx.launch_cache[self.ENTRY_ROWS] = None
+        return x
+
+
+register_stream_op("add_embedding", AddEmbedding)
