@@ -53,9 +53,39 @@ def silu(z):
     return z * torch.sigmoid(z)
 
 
+_NOISE = None      # a function applied to every product's operand rows and result (see ``rounding_noise``), or None
+
+
 def product(x, w, b=None):
-    y = x @ w.T
-    return y if b is None else y + b
+    """x W^T (+ b); with ``_NOISE`` set, rows and result are disturbed as a 16-bit compute type would round them."""
+    if _NOISE is None:
+        y = x @ w.T
+        return y if b is None else y + b
+    y = _NOISE(x) @ w.T
+    return _NOISE(y if b is None else y + b)
+
+
+class rounding_noise:
+    """Inside ``with rounding_noise(seed):`` every product's rows and result are multiplied by 1 + u * 2^-8 with u uniform
+    in (-1, 1), drawn from ``seed``: the relative error of two roundings to bfloat16, at random.  Several seeds show how
+    far the logits of one position move under the compute type's rounding alone; norms, scores, the recurrences' gates
+    and states and the residual stream stay exact, as the design keeps them in 32 bits."""
+
+    def __init__(self, seed: int, amplitude: float = 2.0 ** -8):
+        self.gen = torch.Generator().manual_seed(seed)
+        self.amplitude = amplitude
+
+    def __call__(self, t):
+        return t * (1.0 + (torch.rand(t.shape, generator=self.gen, dtype=t.dtype) * 2.0 - 1.0) * self.amplitude)
+
+    def __enter__(self):
+        global _NOISE
+        _NOISE = self
+        return self
+
+    def __exit__(self, *exc):
+        global _NOISE
+        _NOISE = None
 
 
 def bigram_rows(tokens, buckets: int, mul_prev: int, mul_cur: int):
@@ -234,6 +264,11 @@ def run_order(cfg: dict) -> list:
 def forward(cfg: dict, weights: dict, tokens, dtype=torch.float32, layer_outputs: list | None = None):
     """Logits [T, vocab] of one sequence from its first token on.  ``layer_outputs``: a list that receives the stream
     after every layer run."""
+    with torch.no_grad():
+        return _forward(cfg, weights, tokens, dtype, layer_outputs)
+
+
+def _forward(cfg, weights, tokens, dtype, layer_outputs):
     W = {k: (t.to(dtype) if t.is_floating_point() else t) for k, t in weights.items()}
     eps = float(cfg["norm"]["eps"])
     emb = cfg.get("embedding") or {}
