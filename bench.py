@@ -202,6 +202,65 @@ def run_nesezen(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
     return out
 
 
+def renadra_config(width: int, vocab: int, window: int = 1024) -> dict:
+    """Renadra at sizes that resemble a real model's layers: eight layers [parallel, attention, hgrn2, hgrn2, parallel,
+    attention, hgrn2, attention] of which the first four run twice (twelve layer runs), each with a dense feed-forward of
+    2.75 times the width.  Attention heads of 64 elements on one key head per eight, a window of ``window`` positions (the
+    sigmoid-weighted side keeps the first four positions, caps its scores and rescales its frequencies); beside it linear
+    attention of width / 256 heads with 128 key rows and 256 value columns; gated recurrences of width / 128 heads of 128 x
+    128; a bigram table of 100,003 buckets."""
+    heads = width // 64
+    left = {"heads": heads, "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 64, "mask": {"size": window, "keep_first": 4}, "scale": 0.125,
+            "softcap": 50.0, "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    r_heads = max(1, width // 256)
+    right = {"heads": r_heads, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** (-5 - h) for h in range(r_heads)]}
+    par = {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.9}
+    att = {"heads": heads, "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 64, "mask": {"size": window}, "scale": 0.125,
+           "rot": {"base": 10000.0, "dims": 64}}
+    rec = {"heads": max(1, width // 128), "dim": 128, "vdim": 128}
+    dense = {"kind": "dense", "ff": 11 * width // 4}
+    order = ["parallel", "attention", "hgrn2", "hgrn2", "parallel", "attention", "hgrn2", "attention"]
+    mixers = {"parallel": par, "attention": att, "hgrn2": rec}
+    return {"architecture": "Renadra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 100003, "mul_prev": 31, "mul_cur": 7}},
+            "layers": [{"type": t, "mixer": mixers[t], "mlp": dense} for t in order], "loop": {"start": 0, "stop": 4, "times": 2},
+            "max_positions": 4096, "torch_dtype": "bfloat16"}
+
+
+def run_renadra(dtype: str, context: int, steps: int, warmup: int, widths=(1024, 2048)) -> dict:
+    """Prefill (one prompt of 512 and of 2048 tokens in one step) and decode (1, 8 and 64 requests at ``context``) of
+    Renadra beside the two closest decoders at the same width, twelve layer runs and vocabulary (random weights): Nesezen (a
+    pre-norm block over a float residual stream, windowed attention with capped scores, a recurrence with a state per
+    request) and the Llama decoder."""
+    import torch
+    out = {}
+    for width in widths:
+        models = {
+            "renadra": renadra_config(width, 32000),
+            "nesezen": nesezen_config(width, 32000),
+            "llama": dict(TINYLLAMA, num_hidden_layers=12, hidden_size=width, num_attention_heads=width // 64,
+                          num_key_value_heads=max(1, width // 512), head_dim=64, intermediate_size=11 * width // 4, torch_dtype=dtype),
+        }
+        for name, cfg in models.items():
+            row = {}
+            with tempfile.TemporaryDirectory() as folder:
+                engine = make_engine(cfg, folder, dtype, 64, context)
+                for tokens in (512, PREFILL_TOKENS):
+                    t = time_prefill(engine, tokens, seed=100 + tokens, repeats=4)
+                    row[f"prefill_{tokens}_ms"] = round(t * 1e3, 3)
+                    row[f"prefill_{tokens}_tok_per_s"] = round(tokens / t, 1)
+                for batch in (1, 8, 64):
+                    sec, _ = time_decode(engine, batch, context, steps, warmup, seed=batch)
+                    row[f"decode_b{batch}_ms"] = round(sec * 1e3, 4)
+                    row[f"decode_b{batch}_tok_per_s"] = round(batch / sec, 1)
+                row["weights_millions"] = round(sum(_weights_of(engine.model)) / 1e6, 1)
+                del engine
+                torch.cuda.empty_cache()
+            out[f"{name}_w{width}"] = row
+            print(f"[bench] {name} width {width}: {row}", file=sys.stderr, flush=True)
+    return out
+
+
 def _weights_of(model):
     """Numbers of elements of the tensors the model declares (what a checkpoint of it holds)."""
     out = []
@@ -728,6 +787,9 @@ def main() -> int:
                     "normed queries and keys, routed experts) beside a Llama decoder of the same width and depth, and nothing else")
     ap.add_argument("--nesezen", action="store_true", help="prefill and decode of the Nesezen decoder (windowed attention with capped scores, a "
                     "matrix memory, latent attention, routed experts with a shared one) beside Gudutar and the Llama decoder at equal width and depth, and nothing else")
+    ap.add_argument("--renadra", action="store_true", help="prefill and decode of the Renadra decoder (attention with sigmoid weights beside linear "
+                    "attention, windowed attention with normed values, gated recurrences, a bigram embedding, repeated layers) beside Nesezen and the Llama decoder at equal sizes, instead")
+    ap.add_argument("--widths", default=None, metavar="N,N", help="model widths of --renadra (default 1024,2048)")
     ap.add_argument("--kernels", action="store_true", help="every kernel of a decode step and of a prompt step on its own, with its fraction")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -759,6 +821,12 @@ def main() -> int:
         print(json.dumps({"metric": "Nesezen beside Gudutar and the Llama decoder at equal width, depth and vocabulary (random weights): prefill and decode",
                           "dtype": short, "context": args.context,
                           "models": run_nesezen(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
+        return 0
+    if args.renadra:
+        widths = tuple(int(w) for w in args.widths.split(",")) if args.widths else (1024, 2048)
+        print(json.dumps({"metric": "Renadra beside Nesezen and the Llama decoder at equal width, layer runs and vocabulary (random weights): prefill and decode",
+                          "dtype": short, "context": args.context,
+                          "models": run_renadra(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), widths)}))
         return 0
     if args.workload == "ragged64":
         print(json.dumps({"metric": f"output tokens/s, 64 ragged requests at once, prompts 64-2048 tokens, 256 generated each ({model_name}, random weights)",

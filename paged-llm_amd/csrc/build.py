@@ -151,11 +151,16 @@ USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 256)
 SCORE_TERMS_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 144)
 
 
+# ... and those whose attention library without a softmax (sigmoid weights) it makes.
+SIGMOID_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128)
+
+
 def all_targets() -> list[tuple[str, dict]]:
     """Everything a full build compiles: the common sources plus the usual specialisations."""
     targets: list[tuple[str, dict]] = [(s, {}) for s in COMMON_SOURCES]
     targets += [("attention_mfma.hip", {"HEAD_DIM": d}) for d in USUAL_HEAD_DIMS]
     targets += [("attention_mfma.hip", {"HEAD_DIM": d, "SCORE_TERMS": 1}) for d in SCORE_TERMS_HEAD_DIMS]
+    targets += [("attention_sigmoid.hip", {"HEAD_DIM": d}) for d in SIGMOID_HEAD_DIMS]
     return targets
 
 

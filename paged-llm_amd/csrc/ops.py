@@ -1035,6 +1035,9 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     their keys into partitions, the portions to the prompt kernel (a portion of 512 tokens beside 7 decoded tokens
     at context 8192: 109 us in one launch, 36 us in two; at context 1024: 19 us and 24 us)."""
     bs = k_pages.shape[2]
+    if weights is not None and weights.sigmoid and mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
+        return sigmoid_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim, scale,
+                                 window, weights, terms, ctx.max_q_len)
     if weights is not None and weights.any():
         return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
                                        scale, window, terms=terms, weights=weights)
@@ -1100,6 +1103,26 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                     "16..256 in steps of 16 and groups of at most 64 heads", bs, head_dim, num_heads, num_kv_heads)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window, terms=terms)
+
+
+def sigmoid_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads: int, num_kv_heads: int, head_dim: int,
+                      scale: float, window: int, weights: KeyWeights, terms: ScoreTerms | None, max_q_len: int) -> torch.Tensor:
+    """Attention without a softmax on the matrix cores (bfloat16): a visible key weighs sigmoid(cap(scale q . k) + head_bias),
+    not normalised; visible are the last ``window`` positions (0: all) and the sequence's first ``weights.keep_first``.
+    ``max_q_len`` bounds the queries of one sequence of the step (the launch covers that many per sequence)."""
+    S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
+    weights.checked(num_heads, int(window or 0), q.device)
+    _need(q.dtype == torch.bfloat16 and window >= 0 and max_q_len > 0, "sigmoid attention on the matrix cores: bfloat16, a window or none")
+    _need(terms is None or (terms.slopes is None and terms.sinks is None), "sigmoid weights take a cap of the scores and no other term")
+    T = q.shape[0]
+    out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    sig = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+           c_int, c_int, c_float, c_void_p, c_void_p]
+    _check(_fn("attention_sigmoid.hip", "pllm_sigmoid_attention", {"HEAD_DIM": head_dim}, signature=sig)(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables), block_tables.stride(0),
+        _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, int(max_q_len), num_heads, num_kv_heads, bs, c_float(scale), int(window or 0),
+        weights.keep_first, c_float(terms.cap if terms is not None else 0.0), _ptr(weights.head_bias), _stream()), "sigmoid_attention")
+    return out
 
 
 # ------------------------------------------------------------------------------------------- a residual stream kept in float
