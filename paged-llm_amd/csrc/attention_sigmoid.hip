@@ -18,6 +18,7 @@
 // LDS in wave order.  Weights are float and rounded to bfloat16 for the second product, as the softmax kernels round
 // their probabilities.  Values of keys that no column of the tile may see are zeroed (0 * stale data stays 0).
 #include "common.h"
+#include <type_traits>
 
 using namespace pllm;
 
@@ -44,7 +45,7 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-template <int NCB, int WAVES>
+template <int NCB, int WAVES, bool TWO>
 __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
@@ -106,19 +107,24 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
   const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
   const size_t page_stride = page_elems * num_kv_heads;
 
-  for (int b = wave; b < blocks; b += WAVES) {
-    const bool in_kept = b < blocks_kept;
-    const int n0 = in_kept ? b * 64 : k_lo + (b - blocks_kept) * 64;
-    const int limit = in_kept ? kept : vis_hi;                  // keys of this block at or beyond it are nobody's
-    // ---- all of the block's keys and values are asked for together
-    bf16x8 kreg[4][KSTEPS];
-    bf16x4 vreg4[4][DBLOCKS];
+  // One block = 64 keys = four tiles of 16.  All of a block's keys and values are asked for together, and where the
+  // registers hold two blocks the next one travels while this one is used: a prompt of a few thousand tokens leaves
+  // a SIMD with two wavefronts or fewer, which cannot hide each other's waits for memory.
+  struct KVBlock {
+    bf16x8 k[4][KSTEPS];
+    bf16x4 v[4][DBLOCKS];
     bool on[4];
+    int n0;
+  };
+  auto load_block = [&](KVBlock& blk, int b) {
+    const bool in_kept = b < blocks_kept;
+    blk.n0 = in_kept ? b * 64 : k_lo + (b - blocks_kept) * 64;
+    const int limit = in_kept ? kept : vis_hi;                  // keys of this block at or beyond it are nobody's
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-      const int nk = n0 + kt * 16;
-      on[kt] = nk < limit;                                      // uniform
-      if (!on[kt]) continue;
+      const int nk = blk.n0 + kt * 16;
+      blk.on[kt] = nk < limit;                                  // uniform
+      if (!blk.on[kt]) continue;
       const int page = bt[nk >> bs_shift];
       const int off = nk & (block_size - 1);
       const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
@@ -126,12 +132,17 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
         const int dd = s * 32 + g * 8;
-        kreg[kt][s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(krow + dd) : zero8();
+        blk.k[kt][s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(krow + dd) : zero8();
       }
       const bf16* vrow = v_pages + base + off + g * 4;          // + channel * block_size
 #pragma unroll
-      for (int db = 0; db < DBLOCKS; ++db) vreg4[kt][db] = *reinterpret_cast<const bf16x4*>(vrow + (size_t)(db * 16 + r) * block_size);
+      for (int db = 0; db < DBLOCKS; ++db) blk.v[kt][db] = *reinterpret_cast<const bf16x4*>(vrow + (size_t)(db * 16 + r) * block_size);
     }
+  };
+  // (seen_by_all: every key of the block is visible to every column of a full tile, so nothing is masked)
+  auto compute_block_as = [&](KVBlock& blk, auto seen_by_all) {
+    constexpr bool kAll = decltype(seen_by_all)::value;
+    const int n0 = blk.n0;
     // ---- S^T = K Q^T for four tiles of 16 keys, then the weights; lane holds keys n0 + kt*16 + g*4 + i of its column
     bf16x8 p_op[2][NCB];                                        // B operands of the second product
 #pragma unroll
@@ -139,14 +150,14 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
 #pragma unroll
       for (int cb = 0; cb < NCB; ++cb) {
         floatx4 s_t = floatx4{0.f, 0.f, 0.f, 0.f};
-        if (on[kt]) {
+        if (blk.on[kt]) {
 #pragma unroll
-          for (int s = 0; s < KSTEPS; ++s) s_t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt][s], qreg[cb][s], s_t, 0, 0, 0);
+          for (int s = 0; s < KSTEPS; ++s) s_t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[kt][s], qreg[cb][s], s_t, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int n = n0 + kt * 16 + g * 4 + i;
-          const bool vis = on[kt] && n <= my_qpos[cb] && (n >= my_first[cb] || n < keep_first);
+          const bool vis = kAll || (blk.on[kt] && n <= my_qpos[cb] && (n >= my_first[cb] || n < keep_first));
           float z = capped ? fmaf(-2.f * cap_l2, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s_t[i] * cap_in) + 1.f), cap_l2) : s_t[i] * sl2;
           z += my_bias[cb];
           const float p = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-z));
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
     // ---- O^T += V^T P^T : A operand = 16 channels x 32 keys (k slots 0-3: tile 2a, 4-7: tile 2a+1)
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
-      if (!on[2 * a]) continue;
+      if (!blk.on[2 * a]) continue;
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db) {
         bf16x8 vreg;
@@ -167,14 +178,48 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int n = n0 + kt * 16 + g * 4 + i;
-            const bool anybody = on[kt] && n < vis_hi && (n >= vis_lo || n < keep_first);
-            vreg[h * 4 + i] = anybody ? vreg4[kt][db][i] : (__bf16)0.0f;
+            const bool anybody = kAll || (blk.on[kt] && n < vis_hi && (n >= vis_lo || n < keep_first));
+            vreg[h * 4 + i] = anybody ? blk.v[kt][db][i] : (__bf16)0.0f;
           }
         }
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
           acc[cb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg, p_op[a][cb], acc[cb][db], 0, 0, 0);
       }
+    }
+  };
+  const int first_of_last = first_visible_key(qpos_max, window);
+  const bool full_tile = col0 + 16 * NCB <= num_cols;
+  auto compute_block = [&](KVBlock& blk) {
+    const int n0 = blk.n0;
+    const bool all = full_tile && blk.on[3] && n0 + 63 <= qpos_min && (n0 >= first_of_last || n0 + 64 <= keep_first);
+    if (all) compute_block_as(blk, std::true_type{}); else compute_block_as(blk, std::false_type{});
+  };
+  constexpr bool kTwoBlocks = TWO && 4 * KSTEPS * 4 + 4 * DBLOCKS * 2 <= 64;
+  if constexpr (kTwoBlocks) {
+    KVBlock blk_a, blk_b;
+    int b = wave;
+    if (b < blocks) {
+      load_block(blk_a, b);
+      while (true) {
+        const int b1 = b + WAVES;
+        const bool has1 = b1 < blocks;
+        if (has1) load_block(blk_b, b1);
+        compute_block(blk_a);
+        if (!has1) break;
+        const int b2 = b1 + WAVES;
+        const bool has2 = b2 < blocks;
+        if (has2) load_block(blk_a, b2);
+        compute_block(blk_b);
+        if (!has2) break;
+        b = b2;
+      }
+    }
+  } else {
+    KVBlock blk;
+    for (int b = wave; b < blocks; b += WAVES) {
+      load_block(blk, b);
+      compute_block(blk);
     }
   }
 
@@ -214,32 +259,40 @@ __global__ __launch_bounds__(WAVES * 64) void sigmoid_attention_kernel(
 }
 
 // max_q_len: a bound on the queries of one sequence of this launch (the grid covers that many columns per sequence
-// and kv head; tiles past a sequence's own columns leave at once).  Steps of few columns per kv head (decoding) take
-// one tile of 16 columns and several wavefronts that share the keys; steps with prompt portions tiles of 32 columns
-// (16 for head sizes beyond 64, whose registers two tiles would overflow), one wavefront each.  q, out: rows of heads * D bfloat16 elements with 16-byte aligned strides.
+// and kv head; tiles past a sequence's own columns leave at once).  ncb: tiles of 16 columns per workgroup (1 or 2);
+// waves: wavefronts per workgroup that share its columns and deal its key blocks (1, 2, 4 or 8); two_blocks: the next
+// block's loads are asked for before this block is used (head sizes up to 64).  q, out: rows of heads * D bfloat16
+// elements with 16-byte aligned strides.
 PLLM_API int pllm_sigmoid_attention(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride,
                                     const int* block_tables, int bt_stride, const int* cu_seqlens_q, const int* seq_lens_k,
                                     int num_seqs, int max_q_len, int num_heads, int num_kv_heads, int block_size, float scale,
-                                    int window, int keep_first, float cap, const float* head_bias, hipStream_t stream) {
+                                    int window, int keep_first, float cap, const float* head_bias, int ncb, int waves, int two_blocks,
+                                    hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads || block_size < 16 || (block_size & (block_size - 1)) || window < 0 || keep_first < 0 ||
       !(cap >= 0.f) || (q_stride & 7) || (out_stride & 3) || num_seqs > 65535 || num_kv_heads > 65535)
     return -2;
   const int G = num_heads / num_kv_heads;
   const long cols = (long)max_q_len * G;
-#define PLLM_SIGMOID(NCB, WAVES, LDS)                                                                                                   \
-  hipLaunchKernelGGL((sigmoid_attention_kernel<NCB, WAVES>), dim3((unsigned)((cols + 16 * NCB - 1) / (16 * NCB)), num_kv_heads, num_seqs),  \
-                     dim3(WAVES * 64), LDS, stream, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out,     \
-                     out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, block_size, scale, window,   \
-                     keep_first, cap, head_bias)
-  if (cols <= 16) {
-    constexpr int kWaves = D <= 128 ? 8 : 4;
-    PLLM_SIGMOID(1, kWaves, (size_t)kWaves * DBLOCKS * 4 * 64 * sizeof(float));
-  } else if (D <= 64) {
-    PLLM_SIGMOID(2, 1, 0);
-  } else {
-    PLLM_SIGMOID(1, 1, 0);
+#define PLLM_SIGMOID(NCB, WAVES, TWO)                                                                                                   \
+  hipLaunchKernelGGL((sigmoid_attention_kernel<NCB, WAVES, TWO>), dim3((unsigned)((cols + 16 * NCB - 1) / (16 * NCB)), num_kv_heads, num_seqs), \
+                     dim3(WAVES * 64), WAVES > 1 ? (size_t)WAVES * NCB * DBLOCKS * 4 * 64 * sizeof(float) : 0, stream, (const bf16*)q, q_stride,  \
+                     (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k,     \
+                     num_heads, num_kv_heads, block_size, scale, window, keep_first, cap, head_bias)
+#define PLLM_SIGMOID_WAVES(NCB, TWO)                                       \
+  switch (waves) {                                                          \
+    case 1: PLLM_SIGMOID(NCB, 1, TWO); break;                               \
+    case 2: PLLM_SIGMOID(NCB, 2, TWO); break;                               \
+    case 4: PLLM_SIGMOID(NCB, 4, TWO); break;                               \
+    case 8: PLLM_SIGMOID(NCB, 8, TWO); break;                               \
+    default: return -2;                                                     \
   }
+  if ((size_t)waves * ncb * DBLOCKS * 4 * 64 * sizeof(float) > 64 * 1024 && waves > 1) return -2;
+  if (ncb == 1 && two_blocks) { PLLM_SIGMOID_WAVES(1, true) }
+  else if (ncb == 1) { PLLM_SIGMOID_WAVES(1, false) }
+  else if (ncb == 2 && !two_blocks) { PLLM_SIGMOID_WAVES(2, false) }
+  else return -2;
+#undef PLLM_SIGMOID_WAVES
 #undef PLLM_SIGMOID
   PLLM_RETURN_LAST_ERROR();
 }

@@ -1105,8 +1105,26 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                    num_kv_heads, head_dim, scale, window, terms=terms)
 
 
+def sigmoid_attention_plan(columns: int, head_dim: int, work_items: int = 1) -> tuple:
+    """(tiles of 16 columns per workgroup, wavefronts that share them and deal the key blocks, whether the next block is asked for
+    ahead) for a launch whose sequences have up to ``columns`` (query, head) pairs per kv head; ``work_items``: sequences times
+    kv heads.  Measured at head size 64, 32 heads on 4 key heads, a window of 1,024: a prompt of 2,048 tokens 85 us with one
+    wavefront per 32 columns (90 with two, 100 with four; 101 with tiles of 16 columns; asking for the next block ahead costs
+    registers and gains nothing: 102 to 125); a prompt of 512 tokens 29 / 23 / 17.5 us with one / two / four wavefronts (too few
+    workgroups to fill the GPU otherwise); one decoded token at context 2,048: 14 us with eight wavefronts, 22 with four."""
+    if columns <= 16:
+        return (1, 8 if head_dim <= 128 else 4, False)              # decoding: one tile, the keys split over the wavefronts
+    ncb = 2 if head_dim <= 64 else 1
+    workgroups = -(-columns // (16 * ncb)) * max(1, work_items)
+    waves = 4 if workgroups <= 768 else (2 if workgroups <= 1536 else 1)
+    while waves > 1 and waves * ncb * head_dim * 64 * 4 > 64 * 1024:        # (the wavefronts' outputs meet in LDS)
+        waves //= 2
+    return (ncb, waves, False)
+
+
 def sigmoid_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads: int, num_kv_heads: int, head_dim: int,
-                      scale: float, window: int, weights: KeyWeights, terms: ScoreTerms | None, max_q_len: int) -> torch.Tensor:
+                      scale: float, window: int, weights: KeyWeights, terms: ScoreTerms | None, max_q_len: int,
+                      plan: tuple | None = None) -> torch.Tensor:
     """Attention without a softmax on the matrix cores (bfloat16): a visible key weighs sigmoid(cap(scale q . k) + head_bias),
     not normalised; visible are the last ``window`` positions (0: all) and the sequence's first ``weights.keep_first``.
     ``max_q_len`` bounds the queries of one sequence of the step (the launch covers that many per sequence)."""
@@ -1116,12 +1134,14 @@ def sigmoid_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_
     _need(terms is None or (terms.slopes is None and terms.sinks is None), "sigmoid weights take a cap of the scores and no other term")
     T = q.shape[0]
     out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    ncb, waves, two = plan or sigmoid_attention_plan(max_q_len * (num_heads // num_kv_heads), head_dim, S * num_kv_heads)
     sig = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-           c_int, c_int, c_float, c_void_p, c_void_p]
+           c_int, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p]
     _check(_fn("attention_sigmoid.hip", "pllm_sigmoid_attention", {"HEAD_DIM": head_dim}, signature=sig)(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables), block_tables.stride(0),
         _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, int(max_q_len), num_heads, num_kv_heads, bs, c_float(scale), int(window or 0),
-        weights.keep_first, c_float(terms.cap if terms is not None else 0.0), _ptr(weights.head_bias), _stream()), "sigmoid_attention")
+        weights.keep_first, c_float(terms.cap if terms is not None else 0.0), _ptr(weights.head_bias), ncb, waves, int(two), _stream()),
+        "sigmoid_attention")
     return out
 
 
