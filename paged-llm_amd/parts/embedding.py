@@ -60,6 +60,8 @@ class HashedBigramEmbedding(Part):
         self.buckets, self.mul_prev, self.mul_cur = int(params["buckets"]), int(params["mul_prev"]), int(params["mul_cur"])
         if self.buckets <= 0:
             raise ValueError(f"a bigram table needs a positive number of buckets, got {self.buckets}")
+        # (a b) mod m = ((a mod m) b) mod m: multipliers of any size become numbers below the buckets, and the kernel's products stay small
+        self.mul_prev, self.mul_cur = self.mul_prev % self.buckets, self.mul_cur % self.buckets
         self.tensor_name = params.get("tensor_name", "weight")
         self.pairs_name = params.get("pairs_name", "pairs")
         self.dtype, self.device = env.dtype, env.device
