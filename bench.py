@@ -204,17 +204,17 @@ def run_nesezen(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
 
 def renadra_config(width: int, vocab: int, window: int = 1024) -> dict:
     """Renadra at sizes that resemble a real model's layers: eight layers [parallel, attention, hgrn2, hgrn2, parallel,
-    attention, hgrn2, attention] of which the first four run twice (twelve layer runs), each with a dense feed-forward of
+    attention, hgrn2, attention] of which layers 2 to 5 run twice (twelve layer runs), each with a dense feed-forward of
     2.75 times the width.  Attention heads of 64 elements on one key head per eight, a window of ``window`` positions (the
     sigmoid-weighted side keeps the first four positions, caps its scores and rescales its frequencies); beside it linear
     attention of width / 256 heads with 128 key rows and 256 value columns; gated recurrences of width / 128 heads of 128 x
     128; a bigram table of 100,003 buckets."""
     heads = width // 64
     left = {"heads": heads, "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 64, "mask": {"size": window, "keep_first": 4}, "scale": 0.125,
-            "softcap": 50.0, "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+            "softcap": 50.0, "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}}}
     r_heads = max(1, width // 256)
     right = {"heads": r_heads, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** (-5 - h) for h in range(r_heads)]}
-    par = {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.9}
+    par = {"left": left, "right": right, "left_scale": 1.0, "right_scale": 0.5}
     att = {"heads": heads, "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 64, "mask": {"size": window}, "scale": 0.125,
            "rot": {"base": 10000.0, "dims": 64}}
     rec = {"heads": max(1, width // 128), "dim": 128, "vdim": 128}
@@ -222,8 +222,8 @@ def renadra_config(width: int, vocab: int, window: int = 1024) -> dict:
     order = ["parallel", "attention", "hgrn2", "hgrn2", "parallel", "attention", "hgrn2", "attention"]
     mixers = {"parallel": par, "attention": att, "hgrn2": rec}
     return {"architecture": "Renadra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
-            "embedding": {"scale": 1.0, "bigram": {"buckets": 100003, "mul_prev": 31, "mul_cur": 7}},
-            "layers": [{"type": t, "mixer": mixers[t], "mlp": dense} for t in order], "loop": {"start": 0, "stop": 4, "times": 2},
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 100003, "mul_prev": 131, "mul_cur": 17}},
+            "layers": [{"type": t, "mixer": mixers[t], "mlp": dense} for t in order], "loop": {"start": 2, "stop": 6, "times": 2},
             "max_positions": 4096, "torch_dtype": "bfloat16"}
 
 

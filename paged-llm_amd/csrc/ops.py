@@ -1117,7 +1117,7 @@ def sigmoid_attention_plan(columns: int, head_dim: int, work_items: int = 1) -> 
     ncb = 2 if head_dim <= 64 else 1
     workgroups = -(-columns // (16 * ncb)) * max(1, work_items)
     waves = 4 if workgroups <= 768 else (2 if workgroups <= 1536 else 1)
-    while waves > 1 and waves * ncb * head_dim * 64 * 4 > 64 * 1024:        # (the wavefronts' outputs meet in LDS)
+    while waves > 1 and waves * ncb * head_dim * 64 > 64 * 1024:            # (the wavefronts' outputs meet in LDS: 64 bytes a wavefront, column tile and channel)
         waves //= 2
     return (ncb, waves, False)
 

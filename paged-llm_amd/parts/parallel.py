@@ -61,7 +61,7 @@ class ParallelMixer(Mixer):
     def forward(self, h, ctx, cache, state):
         outs = [m.forward(h, ctx, cache if m.cache_spec() is not None else None, state if m.state_spec() is not None else None)
                 for _, m, _ in self.sides]
-        if any(isinstance(o, torch.Tensor) is False or o.dim() != 2 for o in outs):
+        if any(not isinstance(o, torch.Tensor) or o.dim() != 2 for o in outs):
             raise RuntimeError("mixers side by side return rows (no partial sums)")
         return ops.scaled_sum(outs[0].contiguous(), self.sides[0][2], outs[1].contiguous(), self.sides[1][2])
 

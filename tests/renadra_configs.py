@@ -5,7 +5,7 @@ import copy
 import math
 
 
-def left(heads=4, kv_heads=2, dim=24, size=21, keep_first=3, rot_dims=16, base=1e4, scale=0.3, softcap=20.0, scaling="default"):
+def left(heads=4, kv_heads=2, dim=24, size=21, keep_first=3, rot_dims=16, base=1e4, scale=0.3, softcap=15.0, scaling="default"):
     """The attention side of a parallel mixer: sigmoid weights, values = keys, a window that keeps the first positions."""
     if scaling == "default":
         scaling = {"factor": 4.0, "original": 48, "fast": 8.0, "slow": 1.0}

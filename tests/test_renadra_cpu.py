@@ -88,7 +88,7 @@ def test_rotary_tables_of_the_engine_are_the_plain_ones():
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
     env = BuildEnv(64, torch.float32, torch.device("cpu"), 64, shared={})
-    for dims, base, scaling in ((16, 1e4, {"factor": 4.0, "original": 48, "fast": 8.0, "slow": 1.0}), (40, 100.0, {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}),
+    for dims, base, scaling in ((16, 1e4, {"factor": 4.0, "original": 48, "fast": 8.0, "slow": 1.0}), (40, 100.0, {"factor": 6.0, "original": 512, "fast": 24.0, "slow": 1.5}),
                                 (16, 5e5, {"factor": 16.0, "original": 32, "fast": 4.0, "slow": 0.5}), (10, 33.0, None)):
         engine_scaling = dict(scaling, rope_type="yarn") if scaling else None
         part = RotaryEncoding({"head_dim": 48, "theta": base, "rotary_dim": dims, "scaling": engine_scaling, "exact_frequencies": True}, env)
