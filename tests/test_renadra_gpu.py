@@ -575,6 +575,31 @@ def test_greedy_generation_through_the_engine(folders, name):
                         assert token == int(want[pos].argmax()), (pos, token)
 
 
+def test_preempted_requests_start_again_from_an_empty_state(folders):
+    """A page pool too small for three requests at once: the scheduler preempts the request admitted last (pages and state
+    slot given back, its tokens kept) and computes it again later as a longer prompt, from position 0: from zero states and
+    with no token before, in whatever slot it gets.  Float32: the tokens are the plain implementation's greedy choice all the
+    same."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    folder = folders("A", "float32")
+    vocab = RENA_A["vocab"]
+    prompts = [helpers.random_tokens(n, vocab, 400 + n) for n in (30, 22, 27)]
+    engine = LLMEngine(folder, EngineConfig(dtype="float32", num_gpu_blocks=7, block_size=16, max_num_batched_tokens=32,
+                                            max_num_seqs=3, max_model_len=128))
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True))
+    assert engine.stats.num_preemptions > 0 and sum(o.num_preemptions for o in outs) > 0
+    assert engine.cache_manager.slots.num_free == 3
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 40
+        want = plain_logits(folder, p + o.token_ids)
+        for i, token in enumerate(o.token_ids):
+            row = want[len(p) + i - 1]
+            top2 = np.sort(row)[-2:]
+            if top2[1] - top2[0] > 1e-3 * np.abs(row).max():
+                assert token == int(row.argmax()), (len(p), i)
+
+
 def test_the_replay_program_and_the_command_line(folders, tmp_path):
     folder = folders("B", "float32")
     toks = helpers.random_tokens(30, RENA_B["vocab"], 5)
