@@ -248,8 +248,14 @@ PLLM_API int pllm_round_rows(const float* x, void* rows, long n, hipStream_t str
 // Without a branch the stream's row is src = row_index[r] (or r) and nothing is written to the stream.  The weights
 // are the factors themselves (an architecture that stores them around zero adds the one when it loads them).
 // `rows` has a row stride of its own, so that it may be a part of wider rows.
+// A branch that is the weighted sum of two (two mixers side by side): branch[r][i] = first_scale * branch[r][i] +
+// second_scale * second[r][i], formed where the branch is read.  second null: the branch as it is.
+struct BranchPair {
+  const float* second; float first_scale, second_scale;
+};
+
 template <typename TO>
-__global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restrict__ branch, const float* __restrict__ bias,
+__global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restrict__ branch, const BranchPair pair, const float* __restrict__ bias,
                                                            const float* __restrict__ w_branch, float mult, float* stream,
                                                            const int* __restrict__ row_index, const float* __restrict__ w_next, float eps,
                                                            TO* __restrict__ rows, long rows_stride, int hidden) {
@@ -262,9 +268,10 @@ __global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restri
   float sq = 0.f;
   if (branch) {
     const float* v = branch + (size_t)r * hidden;
+    const float* v2 = pair.second ? pair.second + (size_t)r * hidden : nullptr;
     float bsq = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float f = v[i] + (bias ? bias[i] : 0.f);
+      const float f = (v2 ? pair.first_scale * v[i] + pair.second_scale * v2[i] : v[i]) + (bias ? bias[i] : 0.f);
       row[i] = f;
       bsq = fmaf(f, f, bsq);
     }
@@ -304,7 +311,7 @@ struct ChoiceSum {
 constexpr int kHeldPerThread = 16, kHeldThreads = 256;
 
 template <typename TO, typename TH>
-__global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const float* __restrict__ branch, const ChoiceSum sum,
+__global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const float* __restrict__ branch, const BranchPair pair, const ChoiceSum sum,
                                                                          const float* __restrict__ bias, const float* __restrict__ w_branch,
                                                                          float mult, float* stream, const float* __restrict__ w_next, float eps,
                                                                          TO* __restrict__ rows, long rows_stride, int hidden) {
@@ -320,6 +327,7 @@ __global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const f
     wb[j] = (in && w_branch) ? w_branch[i] : 1.f;
     wn[j] = (in && w_next) ? w_next[i] : 1.f;
     f[j] = (in && !sum.expert_out) ? branch[(size_t)r * hidden + i] : 0.f;
+    if (in && pair.second) f[j] = pair.first_scale * f[j] + pair.second_scale * pair.second[(size_t)r * hidden + i];
   }
   if (sum.expert_out) {
     const TH* own = reinterpret_cast<const TH*>(sum.h) + (size_t)r * sum.ld_h;
@@ -366,14 +374,14 @@ __global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const f
 }
 
 template <typename TO>
-static void launch_sandwich_held(int h_dtype, const float* branch, const ChoiceSum& sum, const float* bias, const float* w_branch, float mult,
+static void launch_sandwich_held(int h_dtype, const float* branch, const BranchPair& pair, const ChoiceSum& sum, const float* bias, const float* w_branch, float mult,
                                  float* stream, const float* w_next, float eps, void* rows, long rows_stride, int num_rows, int hidden,
                                  hipStream_t stream_) {
   if (h_dtype == PLLM_F32)
-    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, float>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, sum, bias, w_branch, mult,
+    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, float>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, pair, sum, bias, w_branch, mult,
                        stream, w_next, eps, (TO*)rows, rows_stride, hidden);
   else
-    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, bf16>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, sum, bias, w_branch, mult,
+    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, bf16>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, pair, sum, bias, w_branch, mult,
                        stream, w_next, eps, (TO*)rows, rows_stride, hidden);
 }
 
@@ -384,20 +392,20 @@ PLLM_API int pllm_rms_sandwich_sum(int out_dtype, int h_dtype, const float* expe
   if (num_rows <= 0) return 0;
   if (hidden <= 0 || hidden > kHeldPerThread * kHeldThreads || !stream || !w_branch || !expert_out || !h || !row_of_pair || !weights || top <= 0) return -2;
   const ChoiceSum sum{expert_out, h, ld_h, row_of_pair, weights, top};
-  if (out_dtype == PLLM_F32) launch_sandwich_held<float>(h_dtype, nullptr, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
-  else launch_sandwich_held<bf16>(h_dtype, nullptr, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+  if (out_dtype == PLLM_F32) launch_sandwich_held<float>(h_dtype, nullptr, BranchPair{nullptr, 1.f, 1.f}, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+  else launch_sandwich_held<bf16>(h_dtype, nullptr, BranchPair{nullptr, 1.f, 1.f}, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
   PLLM_RETURN_LAST_ERROR();
 }
 
-PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* bias, const float* w_branch, float mult, float* stream,
-                               const int* row_index, const float* w_next, float eps, void* rows, long rows_stride, int num_rows,
-                               int hidden, hipStream_t stream_) {
+static int rms_sandwich_launch(int out_dtype, const float* branch, const BranchPair pair, const float* bias, const float* w_branch, float mult,
+                               float* stream, const int* row_index, const float* w_next, float eps, void* rows, long rows_stride,
+                               int num_rows, int hidden, hipStream_t stream_) {
   if (num_rows <= 0) return 0;
   if (hidden <= 0 || !stream) return -2;
   if (branch && hidden <= kHeldPerThread * kHeldThreads) {
     const ChoiceSum none{nullptr, nullptr, 0, nullptr, nullptr, 0};
-    if (out_dtype == PLLM_F32) launch_sandwich_held<float>(PLLM_F32, branch, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
-    else launch_sandwich_held<bf16>(PLLM_F32, branch, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+    if (out_dtype == PLLM_F32) launch_sandwich_held<float>(PLLM_F32, branch, pair, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+    else launch_sandwich_held<bf16>(PLLM_F32, branch, pair, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
     PLLM_RETURN_LAST_ERROR();
   }
   const size_t lds = (size_t)(hidden + 16) * sizeof(float);
@@ -409,12 +417,28 @@ PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* 
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                          \
       if (e != hipSuccess) return (int)e;                                                                                 \
     }                                                                                                                     \
-    hipLaunchKernelGGL(rms_sandwich_kernel<TO>, grid, block, lds, stream_, branch, bias, w_branch, mult, stream, row_index, \
+    hipLaunchKernelGGL(rms_sandwich_kernel<TO>, grid, block, lds, stream_, branch, pair, bias, w_branch, mult, stream, row_index, \
                        w_next, eps, (TO*)rows, rows_stride, hidden);                                                      \
   } while (0)
   if (out_dtype == PLLM_F32) PLLM_SW(float); else PLLM_SW(bf16);
 #undef PLLM_SW
   PLLM_RETURN_LAST_ERROR();
+}
+
+PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* bias, const float* w_branch, float mult, float* stream,
+                               const int* row_index, const float* w_next, float eps, void* rows, long rows_stride, int num_rows,
+                               int hidden, hipStream_t stream_) {
+  return rms_sandwich_launch(out_dtype, branch, BranchPair{nullptr, 1.f, 1.f}, bias, w_branch, mult, stream, row_index, w_next, eps, rows,
+                             rows_stride, num_rows, hidden, stream_);
+}
+
+// The same with a branch that is first_scale * branch + second_scale * second (both float rows like the stream).
+PLLM_API int pllm_rms_sandwich_pair(int out_dtype, const float* branch, float first_scale, const float* second, float second_scale,
+                                    const float* bias, const float* w_branch, float mult, float* stream, const float* w_next, float eps,
+                                    void* rows, long rows_stride, int num_rows, int hidden, hipStream_t stream_) {
+  if (!branch || !second) return -2;
+  return rms_sandwich_launch(out_dtype, branch, BranchPair{second, first_scale, second_scale}, bias, w_branch, mult, stream, nullptr, w_next,
+                             eps, rows, rows_stride, num_rows, hidden, stream_);
 }
 
 // ---------------------------------------------------------------------------------------------

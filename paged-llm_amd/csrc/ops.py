@@ -1625,6 +1625,20 @@ class ChoiceSum:
         return e, h, rp, wt
 
 
+class WeightedPair:
+    """A branch that is the weighted sum of two, first_scale * first + second_scale * second (contiguous float32 rows of one
+    shape: two mixers side by side), which the kernel that adds the branch to the stream forms where it reads it
+    (``rms_sandwich``).  ``rows()`` forms it for any other reader."""
+
+    __slots__ = ("first", "first_scale", "second", "second_scale")
+
+    def __init__(self, first: torch.Tensor, first_scale: float, second: torch.Tensor, second_scale: float):
+        self.first, self.first_scale, self.second, self.second_scale = first, float(first_scale), second, float(second_scale)
+
+    def rows(self) -> torch.Tensor:
+        return scaled_sum(self.first, self.first_scale, self.second, self.second_scale)
+
+
 def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: torch.Tensor | None, mult: float, eps: float,
                  w_next: torch.Tensor | None = None, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
                  bias: torch.Tensor | None = None, row_index: torch.Tensor | None = None) -> torch.Tensor | None:
@@ -1635,6 +1649,8 @@ def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: to
     rows of the stream as it is now are returned in that type: normed and times ``w_next``, or as they are when
     ``w_next`` is None.  ``out`` may be a view with a row stride of its own (unit inner stride).  Without a branch
     ``row_index`` (int32) picks the rows of the stream; nothing is written to the stream then."""
+    if isinstance(branch, WeightedPair):
+        return _rms_sandwich_pair(stream, branch, w_branch, mult, eps, w_next, out, out_dtype, bias, row_index)
     _on_gpu(stream, None if isinstance(branch, ChoiceSum) else branch, w_branch, w_next, out, bias, row_index)
     _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
     rows, H = stream.shape
@@ -1686,6 +1702,28 @@ def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float) -> torch.
     return out
 
 
+def _rms_sandwich_pair(stream, pair: WeightedPair, w_branch, mult, eps, w_next, out, out_dtype, bias, row_index):
+    _on_gpu(stream, pair.first, pair.second, w_branch, w_next, out, bias)
+    _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
+    rows, H = stream.shape
+    _need((H + 16) * 4 <= min(_max_lds_bytes(stream.device), 160 * 1024), f"the norm kernel stages one row in LDS: hidden size {H} is above its limit")
+    _need(row_index is None, "rows are picked only where no branch is added")
+    for t in (pair.first, pair.second):
+        _need(t.dtype == torch.float32 and t.shape == stream.shape and t.is_contiguous(), "a pair's branches are contiguous float32 rows like the stream")
+    for t, what in ((w_branch, "w_branch"), (w_next, "w_next"), (bias, "bias")):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()), f"{what} must be float32 [{H}]")
+    if out is None and out_dtype is not None:
+        out = torch.empty((rows, H), dtype=out_dtype, device=stream.device)
+    if out is not None:
+        _need(out.dim() == 2 and out.shape == (rows, H) and out.stride(1) == 1, f"the rows' output is [{rows}, {H}] with unit inner stride")
+    sig = [c_int, c_void_p, c_float, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_void_p]
+    _check(_fn("float_stream.hip", "pllm_rms_sandwich_pair", signature=sig)(
+        dtype_code(out.dtype) if out is not None else F32, _ptr(pair.first), c_float(pair.first_scale), _ptr(pair.second), c_float(pair.second_scale),
+        _ptr(bias), _ptr(w_branch), c_float(mult), _ptr(stream), _ptr(w_next), c_float(eps), _ptr(out), out.stride(0) if out is not None else 0,
+        rows, H, _stream()), "rms_sandwich_pair")
+    return out
+
+
 def place_rows(x: torch.Tensor, out: torch.Tensor) -> None:
     """out[:, :] = x converted to out's type; x contiguous float32 [rows, hidden], out a view [rows, hidden] of wider rows."""
     _on_gpu(x, out)
@@ -1700,6 +1738,8 @@ def dynamic_tanh(stream: torch.Tensor, alpha: float, weight: torch.Tensor | None
     """Around a float32 residual stream [rows, hidden]: with ``branch`` (float32 rows like the stream, or a ``ChoiceSum``: a
     weighted sum of experts' rows that the kernel forms itself) stream += branch in place; then, when ``out_dtype`` is given, the rows tanh(alpha * stream) * weight + bias of the stream as it is now are
     returned in that type (``row_index``, int32, picks rows when no branch is added)."""
+    if isinstance(branch, WeightedPair):
+        branch = branch.rows()
     _on_gpu(stream, weight, bias, None if isinstance(branch, ChoiceSum) else branch, row_index)
     _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
     rows, H = stream.shape

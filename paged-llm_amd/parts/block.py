@@ -209,7 +209,11 @@ class FloatPreNormBlock(Block):
         after = getattr(ctx, "next_entry_norm", None)
         after = after if hasattr(after, "sum_then") else None
         ctx.partial_sums_ok, ctx.float_branch = False, True
+        # a mixer made of two may hand over their weighted sum unformed (``ops.WeightedPair``) when the kernel behind it forms it
+        reader = p["feed_forward_norm"] if self.has_feed_forward else after
+        ctx.branch_pair_ok = bool(getattr(reader, "takes_weighted_pair", False))
         a = p["mixer"].forward(self._entry_rows(x, ctx), ctx, cache, state)
+        ctx.branch_pair_ok = False
         if self.has_feed_forward:
             h = p["feed_forward_norm"].sum_then(x, a)
             ctx.branch_sum_ok = True      # a feed-forward may hand over a sum that the kernel behind it forms (``ops.ChoiceSum``)

@@ -123,12 +123,14 @@ class RMSNorm(Norm):
         return ops.rms_sandwich(stream, branch, self.weight, mult, self.eps, w_next=then.weight if then is not None else None,
                                 out=out, out_dtype=self.dtype if want_rows and out is None else None, bias=bias)
 
+    takes_weighted_pair = True          # ``sum_then`` forms a branch that is the weighted sum of two (``ops.WeightedPair``) in its kernel
+
     def sum_then(self, stream: torch.Tensor, branch) -> torch.Tensor:
         """stream += branch in place (float, the branch as it is); returns this norm's rows of the new stream in the compute
         type, from the same kernel (a pre-norm block over a float stream)."""
         if isinstance(branch, ops.ChoiceSum):
             branch = branch.rows()
-        return ops.rms_sandwich(stream, branch, None, 1.0, self.eps, w_next=self.weight, out_dtype=self.dtype)
+        return ops.rms_sandwich(stream, branch, None, 1.0, self.eps, w_next=self.weight, out_dtype=self.dtype)      # (a ``WeightedPair`` is formed by the kernel)
 
     def add_norm(self, x, delta, row_index=None, write_residual=True):
         return ops.rmsnorm(x, self.weight, self.eps, delta, row_index, write_residual)

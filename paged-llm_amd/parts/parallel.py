@@ -5,7 +5,8 @@
 Each side is any registered mixer with parameters of its own; its tensors lie under the side's prefix (``left.*``,
 ``right.*``).  One side at most keeps pages and one side at most keeps a state of fixed size per request (the layer's
 cache and its state slot are handed to whichever side declared them), so attention beside a recurrence is served by
-the cache manager and the state slots as each alone would be.
+the cache manager and the state slots as each alone would be.  Under a block whose sum-and-norm kernel takes it
+(``ctx.branch_pair_ok``) the weighted sum is handed on unformed (``ops.WeightedPair``) and that kernel forms it.
 """
 
 from __future__ import annotations
@@ -63,7 +64,10 @@ class ParallelMixer(Mixer):
                 for _, m, _ in self.sides]
         if any(not isinstance(o, torch.Tensor) or o.dim() != 2 for o in outs):
             raise RuntimeError("mixers side by side return rows (no partial sums)")
-        return ops.scaled_sum(outs[0].contiguous(), self.sides[0][2], outs[1].contiguous(), self.sides[1][2])
+        a, b = outs[0].contiguous(), outs[1].contiguous()
+        if getattr(ctx, "branch_pair_ok", False) and a.dtype == torch.float32 and b.dtype == torch.float32:
+            return ops.WeightedPair(a, self.sides[0][2], b, self.sides[1][2])        # formed by the kernel that adds it to the stream
+        return ops.scaled_sum(a, self.sides[0][2], b, self.sides[1][2])
 
 
 register_mixer("parallel", ParallelMixer)

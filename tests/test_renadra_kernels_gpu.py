@@ -258,3 +258,13 @@ def test_pre_norm_sum_in_the_rms_kernel(hidden, out_dtype):
     assert torch.allclose(got.float().cpu(), s / torch.sqrt((s * s).mean(-1, keepdim=True) + 1e-5) * w, atol=tol, rtol=tol)
     a, b = dev(x), dev(d)
     assert torch.allclose(ops.scaled_sum(a, 0.8, b, -1.25).cpu(), 0.8 * x - 1.25 * d, atol=1e-6)
+    # a branch that is the weighted sum of two, formed by the same kernel
+    e = randn(5, hidden, seed=4)
+    stream = dev(x.clone())
+    got = ops.rms_sandwich(stream, ops.WeightedPair(dev(d), 0.7, dev(e), 1.2), None, 1.0, 1e-5, w_next=dev(w), out_dtype=out_dtype)
+    s = x + (0.7 * d + 1.2 * e)
+    assert torch.allclose(stream.cpu(), s, atol=1e-6, rtol=1e-6)
+    assert torch.allclose(got.float().cpu(), s / torch.sqrt((s * s).mean(-1, keepdim=True) + 1e-5) * w, atol=tol, rtol=tol)
+    stream = dev(x.clone())
+    ops.stream_add(stream, ops.WeightedPair(dev(d), 0.7, dev(e), 1.2))
+    assert torch.allclose(stream.cpu(), s, atol=1e-6, rtol=1e-6)
